@@ -1,0 +1,265 @@
+/*
+ * tlf_hip.h - C ABI of libtlf_hip.so: the per-token hot path of a TinyLLMForge
+ * (tinyvllm) engine as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions (all entry points):
+ *   - extern "C", plain pointers and sizes; no C++ or torch types.
+ *   - Every pointer is a DEVICE pointer owned by the caller (the reference lets
+ *     PyTorch own every buffer, so the binding passes tensor.data_ptr()).
+ *   - The last argument is a hipStream_t passed as void*; work is only enqueued
+ *     on that stream.  No entry point allocates, frees, synchronises or reads
+ *     device memory on the host, so every call can be stream-captured into a
+ *     hipGraph.  Launch geometry depends only on the integer arguments, never
+ *     on device data.
+ *   - Return value: 0 = ok, < 0 = rejected argument (TLF_E_*), > 0 = hipError_t
+ *     of the failed launch.  Nothing is launched when an argument is rejected.
+ *   - "bf16" is bfloat16 stored as uint16; "rows" are tokens unless said otherwise.
+ *   - Scratch memory is caller provided: ask tlf_*_workspace_bytes() and pass a
+ *     buffer of at least that size (256-byte aligned).
+ *
+ * Each declaration cites the reference interface (file:line under the
+ * reference's tinyvllm/ package) that it replaces.
+ */
+#ifndef TLF_HIP_H
+#define TLF_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TLF_ABI_VERSION 1
+
+#define TLF_OK 0
+#define TLF_E_NULL (-1)        /* a required pointer is NULL                         */
+#define TLF_E_SHAPE (-2)       /* a size is negative, zero where not allowed, or unsupported */
+#define TLF_E_ALIGN (-3)       /* a pointer or stride breaks the stated alignment    */
+#define TLF_E_WORKSPACE (-4)   /* workspace missing or too small                     */
+#define TLF_E_UNSUPPORTED (-5) /* a combination this build has no kernel for          */
+
+/* KV-cache element types */
+#define TLF_KV_BF16 0
+#define TLF_KV_FP8_E4M3 1 /* OCP e4m3fn, per-KV-head fp32 scale */
+
+/* ABI version of the loaded library (== TLF_ABI_VERSION it was built with). */
+int tlf_version(void);
+/* Static, human readable text for a return code of this library. */
+const char *tlf_error_string(int code);
+/* Multiprocessor count and LDS bytes per workgroup of the current device
+ * (host query; either out pointer may be NULL). */
+int tlf_device_info(int32_t *num_cus, int32_t *lds_bytes);
+
+/* ---------------------------------------------------------------------------
+ * a1  store_kvcache   replaces layers/attention.py:33-48 (Triton kernel 9-30)
+ *
+ *   cache_row(slot[i]) = key[i] / value[i]  for every token i with slot[i] >= 0
+ *
+ * key/value: [num_tokens, row_bytes] rows, 16-byte aligned, row strides in
+ * BYTES (value is a strided view into the qkv projection in the reference,
+ * models/qwen3.py:79).  k_cache/v_cache: [num_slots, row_bytes] contiguous
+ * (= [nblk, block_size, Hkv, Dh]).  row_bytes % 16 == 0.  A negative slot is
+ * skipped (graph padding rows); slot >= num_slots is also skipped, never
+ * written.  Pure byte copy: exact for any element type.
+ */
+int tlf_store_kvcache(const void *key, int64_t key_stride_bytes,
+                      const void *value, int64_t value_stride_bytes,
+                      void *k_cache, void *v_cache,
+                      const int32_t *slot_mapping, int32_t num_tokens,
+                      int32_t row_bytes, int64_t num_slots, void *stream);
+
+/* a13 (build-defined, no reference counterpart): bf16 rows -> e4m3 cache rows,
+ * c = e4m3(sat(x / scale[h])).  key/value rows are [Hkv, Dh] bf16 (strides in
+ * bytes), cache rows are Hkv*Dh bytes.  k_scale/v_scale: fp32 [Hkv].  Dh % 8 == 0. */
+int tlf_store_kvcache_fp8(const void *key, int64_t key_stride_bytes,
+                          const void *value, int64_t value_stride_bytes,
+                          void *k_cache, void *v_cache,
+                          const int32_t *slot_mapping, int32_t num_tokens,
+                          int32_t num_kv_heads, int32_t head_dim,
+                          const float *k_scale, const float *v_scale,
+                          int64_t num_slots, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * a5  RMSNorm.rms_forward   replaces layers/layernorm.py:21-31
+ *
+ *   y = bf16( bf16( x * rsqrt(mean(x^2) + eps) ) * w )      (fp32 math)
+ *
+ * x is viewed as [outer, inner, cols] bf16 with element strides
+ * (x_outer_stride, cols, 1): the q/k-norm call normalises every head of a
+ * strided slice of the qkv projection (models/qwen3.py:80-83), the layer norm
+ * uses inner = 1.  y is [outer, inner, cols] contiguous.  cols % 8 == 0,
+ * cols <= 16384, 16-byte aligned rows.
+ */
+int tlf_rmsnorm(const void *x, int64_t x_outer_stride, const void *weight, void *y,
+                int32_t outer, int32_t inner, int32_t cols, float eps, void *stream);
+
+/* a6  RMSNorm.add_rms_forward   replaces layers/layernorm.py:33-45
+ *
+ *   s = x + residual (fp32); residual_out = bf16(s);
+ *   y = bf16( bf16( s * rsqrt(mean(s^2) + eps) ) * w )
+ *
+ * All [rows, cols] bf16 contiguous.  y may alias x and residual_out may alias
+ * residual (each thread reads its elements before writing them).
+ */
+int tlf_add_rmsnorm(const void *x, const void *residual, const void *weight,
+                    void *y, void *residual_out,
+                    int32_t rows, int32_t cols, float eps, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * a7  RotaryEmbedding.forward   replaces layers/rotary_embedding.py:41-57 (+5-15)
+ *
+ *   cs = cos_sin[positions[i]]  (fp32 [max_pos, head_dim] = cos || sin)
+ *   per head: y[:d/2] = cos*x[:d/2] - sin*x[d/2:], y[d/2:] = cos*x[d/2:] + sin*x[:d/2]
+ *   (neox half split, fp32 products rounded separately, one bf16 rounding)
+ *
+ * q: [n, num_q_heads*head_dim] bf16 with row stride q_stride (elements), k
+ * likewise; outputs contiguous and may alias the inputs.  positions int64 [n],
+ * each in [0, max_pos) (rows with a position outside the table are left
+ * untouched).  head_dim % 16 == 0.
+ */
+int tlf_rope(const int64_t *positions, const void *q, int64_t q_stride,
+             const void *k, int64_t k_stride, const float *cos_sin,
+             void *q_out, void *k_out, int32_t n, int32_t num_q_heads,
+             int32_t num_kv_heads, int32_t head_dim, int32_t max_pos, void *stream);
+
+/* Fused form of the reference's op sequence models/qwen3.py:79-94 +
+ * layers/attention.py:94-95: q/k RMSNorm over head_dim (a5), RoPE (a7) and the
+ * KV-cache store (a1; bf16 or e4m3 by kv_dtype) in one pass over the qkv
+ * projection [n, (Hq + 2 Hkv) * head_dim] (row stride qkv_stride elements).
+ * Writes q_out [n, Hq*head_dim] contiguous; k/v go only to the caches when
+ * slot_mapping is non-NULL, and k_out/v_out (contiguous, may be NULL) receive
+ * the rotated K and the V rows for the prefill attention.  Every intermediate
+ * rounding of the unfused sequence is kept, so results are bit-identical to
+ * running tlf_rmsnorm, tlf_rope and tlf_store_kvcache one after the other.
+ * head_dim == 128.
+ */
+int tlf_qknorm_rope_store(const void *qkv, int64_t qkv_stride,
+                          const void *q_norm_weight, const void *k_norm_weight, float eps,
+                          const int64_t *positions, const float *cos_sin, int32_t max_pos,
+                          void *q_out, void *k_out, void *v_out,
+                          void *k_cache, void *v_cache, const int32_t *slot_mapping,
+                          int64_t num_slots, int32_t kv_dtype,
+                          const float *k_scale, const float *v_scale,
+                          int32_t n, int32_t num_q_heads, int32_t num_kv_heads,
+                          int32_t head_dim, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * a8  SiluAndMul.forward   replaces layers/activation.py:11-14
+ *
+ *   y = bf16( bf16(silu(x[:, :I])) * x[:, I:] )      x [rows, 2I] -> y [rows, I]
+ *
+ * bf16, contiguous, I % 8 == 0.
+ */
+int tlf_silu_and_mul(const void *x, void *y, int32_t rows, int32_t inter, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * a9  Sampler.forward, greedy branch   replaces layers/sampler.py:13-14,21
+ *
+ *   out[b] = first index of max(logits[b, :])       logits bf16 [rows, vocab]
+ *
+ * (bf16 -> fp32 is monotone, so the argmax over bf16 equals the reference's
+ * argmax over the fp32 cast; -0 == +0; NaN logits are not supported.)
+ * out: int64 [rows].  logits row stride in elements.  Needs a workspace.
+ */
+size_t tlf_argmax_workspace_bytes(int32_t rows, int32_t vocab);
+int tlf_argmax(const void *logits, int64_t row_stride, int64_t *out,
+               int32_t rows, int32_t vocab, void *workspace, size_t workspace_bytes,
+               void *stream);
+
+/* ---------------------------------------------------------------------------
+ * a10  weight-only int8 linear (build-defined; the reference has bf16 F.linear
+ * only: layers/linear.py:48-49, 82-83, 180-181; same [N, K] weight layout)
+ *
+ *   y[m, n] = bf16( (sum_k x[m, k] * float(wq[n, k])) * scale[n] )   fp32 accumulate
+ *
+ * x: bf16 [M, K] row stride x_stride (elements); wq: int8 [N, K] contiguous;
+ * scale: fp32 [N]; y: bf16 [M, N] contiguous.  K % 64 == 0, N % 16 == 0.
+ */
+size_t tlf_w8a16_gemm_workspace_bytes(int32_t M, int32_t N, int32_t K);
+int tlf_w8a16_gemm(const void *x, int64_t x_stride, const void *wq, const float *scale,
+                   void *y, int32_t M, int32_t N, int32_t K,
+                   void *workspace, size_t workspace_bytes, void *stream);
+
+/* a10 / f1  bf16 linear   replaces layers/linear.py:48-49, 82-83, 180-181 and the
+ * logits product layers/embed_head.py:63
+ *
+ *   y[m, n] = bf16( sum_k x[m, k] * w[n, k] )      fp32 accumulate
+ *
+ * Same shapes and constraints as tlf_w8a16_gemm with w bf16 [N, K].
+ */
+int tlf_bf16_gemm(const void *x, int64_t x_stride, const void *w, void *y,
+                  int32_t M, int32_t N, int32_t K,
+                  void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * a3  paged decode attention   replaces the decode branch layers/attention.py:106-109
+ *     (flash_attn_with_kvcache, one query token per sequence)
+ *
+ *   out[b, h] = softmax(scale * q[b, h] . K_b^T) V_b    over rows 0..context_lens[b]-1,
+ *   row t of sequence b = cache[block_tables[b, t / block_size], t % block_size, h / (Hq/Hkv), :]
+ *
+ * q: bf16 [batch, Hq, Dh] with row stride q_stride (elements); caches
+ * [num_cache_blocks, block_size, Hkv, Dh] contiguous, bf16 or e4m3 (kv_dtype;
+ * e4m3 rows are dequantised as float(c) * scale[kvh], k_scale/v_scale fp32 [Hkv],
+ * NULL for bf16); block_tables int32 [batch, max_blocks] with row stride
+ * block_table_stride; entries at or beyond ceil(context_len / block_size) are
+ * never dereferenced (the reference pads them with -1 or 0); entries outside
+ * [0, num_cache_blocks) inside that range make the kernel skip the block.
+ * context_lens int32 [batch]; a sequence with context_len <= 0 gets zeros.
+ * out: bf16 [batch, Hq*Dh] contiguous.  fp32 softmax and accumulation, bf16
+ * probabilities in the P.V product (as flash-attn does).
+ * Dh == 128, Hq % Hkv == 0, Hq/Hkv <= 16, Hkv <= 16, block_size % 16 == 0.
+ */
+size_t tlf_paged_decode_attn_workspace_bytes(int32_t batch, int32_t num_q_heads,
+                                             int32_t head_dim, int32_t max_blocks,
+                                             int32_t block_size);
+int tlf_paged_decode_attn(const void *q, int64_t q_stride,
+                          const void *k_cache, const void *v_cache, int32_t kv_dtype,
+                          const float *k_scale, const float *v_scale,
+                          const int32_t *block_tables, int64_t block_table_stride,
+                          const int32_t *context_lens, void *out,
+                          int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
+                          int32_t head_dim, int32_t block_size, int32_t max_blocks,
+                          int64_t num_cache_blocks, float scale,
+                          void *workspace, size_t workspace_bytes, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * a4  varlen causal prefill attention   replaces the prefill branch
+ *     layers/attention.py:96-105 (flash_attn_varlen_func, causal=True)
+ *
+ * q: bf16 [total_q, Hq, Dh] row stride q_stride (elements).  Sequence s owns
+ * query rows cu_seqlens_q[s]..cu_seqlens_q[s+1]-1 and keys
+ * 0..len_k-1 with len_k = cu_seqlens_k[s+1] - cu_seqlens_k[s].  The causal mask
+ * is bottom-right aligned: query i sees keys 0..(len_k - len_q) + i.
+ *   block_tables == NULL: k/v are packed rows [total_k, Hkv, Dh] with row
+ *     strides k_stride/v_stride (elements; v is a strided view in the reference).
+ *   block_tables != NULL: k/v are the paged caches (layout and kv_dtype as in
+ *     tlf_paged_decode_attn) and EVERY sequence reads its keys from them
+ *     (layers/attention.py:99-100).
+ * out: bf16 [total_q, Hq*Dh] contiguous.  max_seqlen_q bounds the grid.
+ * Dh == 128, Hq % Hkv == 0.
+ */
+int tlf_varlen_prefill_attn(const void *q, int64_t q_stride,
+                            const void *k, int64_t k_stride,
+                            const void *v, int64_t v_stride, int32_t kv_dtype,
+                            const float *k_scale, const float *v_scale,
+                            const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k,
+                            const int32_t *block_tables, int64_t block_table_stride,
+                            void *out, int32_t num_seqs, int32_t max_seqlen_q,
+                            int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                            int32_t block_size, int64_t num_cache_blocks, float scale,
+                            void *stream);
+
+/* ---------------------------------------------------------------------------
+ * K9  embedding row gather   replaces layers/embed_head.py:38 (F.embedding)
+ *   y[i] = weight[ids[i]]   ids int64 [n], weight bf16 [vocab, cols], cols % 8 == 0.
+ *   Rows with an id outside [0, vocab) are zero filled.
+ */
+int tlf_embedding(const int64_t *ids, const void *weight, void *y,
+                  int32_t n, int32_t vocab, int32_t cols, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TLF_HIP_H */

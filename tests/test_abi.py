@@ -1,0 +1,60 @@
+"""CPU-side checks of the C-ABI library: it loads and exports every declared symbol.
+
+No compute call is made here (there is no GPU in the build container).
+"""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "tlf_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tlf_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    syms = declared_symbols()
+    for name in ["tlf_store_kvcache", "tlf_paged_decode_attn", "tlf_varlen_prefill_attn", "tlf_rmsnorm",
+                 "tlf_add_rmsnorm", "tlf_rope", "tlf_silu_and_mul", "tlf_argmax", "tlf_w8a16_gemm"]:
+        assert name in syms
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    from tinyllmforge_amd import _lib
+    assert os.path.exists(_lib.LIB_PATH), "build the library first: python tinyllmforge_amd/csrc/build.py"
+    lib = _lib.load()
+    for name in declared_symbols():
+        assert hasattr(lib, name), f"{name} declared in tlf_hip.h but not exported"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature"
+    assert sorted(_lib.SIGNATURES) == declared_symbols()
+    assert lib.tlf_version() == _lib.ABI_VERSION
+    assert lib.tlf_error_string(0) == b"ok"
+    assert b"NULL" in lib.tlf_error_string(-1)
+
+
+def test_argument_rejection_happens_before_any_launch():
+    """NULL pointers / bad shapes are rejected on the host; nothing touches a GPU."""
+    from tinyllmforge_amd import _lib
+    lib = _lib.load()
+    assert lib.tlf_store_kvcache(None, 0, None, 0, None, None, None, 4, 2048, 10, None) == -1
+    assert lib.tlf_store_kvcache(None, 0, None, 0, None, None, None, 0, 2048, 10, None) == 0   # empty batch
+    assert lib.tlf_silu_and_mul(16, 16, 3, 12, None) == -2        # inter % 8 != 0
+    assert lib.tlf_silu_and_mul(8, 16, 3, 16, None) == -3         # misaligned x
+    assert lib.tlf_rmsnorm(16, 128, 16, 16, 2, 1, 100, 1e-6, None) == -2
+    assert lib.tlf_argmax(16, 64, 16, 2, 64, None, 0, None) == -4
+    assert lib.tlf_paged_decode_attn(16, 4096, 16, 16, 0, None, None, 16, 16, 16, 16,
+                                     2, 32, 8, 64, 256, 16, 10, 0.1, None, 0, None) == -5  # Dh != 128
+    assert lib.tlf_argmax_workspace_bytes(4, 151936) > 0
+
+
+def test_ops_refuse_cpu_tensors():
+    import torch
+    from tinyllmforge_amd import ops, _lib
+    with pytest.raises(_lib.TlfError):
+        ops.silu_and_mul(torch.zeros(2, 16, dtype=torch.bfloat16))

@@ -1,0 +1,212 @@
+"""GPU parity: elementwise / row kernels and the KV-cache store against the CPU oracle.
+
+Integer and byte work must be bit-exact.  Floating-point ops follow the oracle's
+rounding points; the only freedom left is the fp32 summation order and the last
+ulp of exp/rsqrt, so results must agree within one bf16 ulp and be bit-identical
+for nearly every element (the thresholds are stated in each test).
+"""
+import pytest
+import torch
+
+from oracle import ops as O
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+DEV = "cuda"
+
+
+def g(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def assert_close_bf16(got, ref, max_ulp=1.0, min_exact=0.995):
+    got, ref = got.float().cpu(), ref.float().cpu()
+    assert got.shape == ref.shape
+    ulp = O.bf16_ulp(ref)
+    err = (got - ref).abs()
+    assert (err <= max_ulp * ulp + 1e-30).all(), f"max err {err.max().item()} ulps {(err / ulp).max().item()}"
+    exact = (got == ref).float().mean().item()
+    assert exact >= min_exact, f"only {exact:.5f} of elements bit-identical"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from tinyllmforge_amd import ops as P
+    return P
+
+
+# ----------------------------------------------------------------------------- a1
+@pytest.mark.parametrize("N,Hkv,Dh,nblk,bs", [(1, 8, 128, 4, 256), (300, 8, 128, 3, 256), (77, 2, 64, 5, 16),
+                                             (4096, 8, 128, 20, 256)])
+def test_store_kvcache_bit_exact(ops, N, Hkv, Dh, nblk, bs):
+    D = Hkv * Dh
+    qkv = torch.randn(N, 3 * D + 128, generator=g(N)).to(BF)
+    key = qkv[:, 128:128 + D].contiguous().view(N, Hkv, Dh)
+    value = qkv[:, 128 + 2 * D:].view(N, Hkv, Dh)                 # strided view, like the qkv split
+    slots = torch.randperm(nblk * bs, generator=g(N + 1))[:N].to(torch.int32)
+    if N > 4:
+        slots[3] = -1                                             # padding row must be skipped
+    kc = torch.randn(nblk, bs, Hkv, Dh, generator=g(5)).to(BF)
+    vc = torch.randn(nblk, bs, Hkv, Dh, generator=g(6)).to(BF)
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    O.store_kvcache(key, value, kc_ref, vc_ref, slots)
+    qkv_d = qkv.to(DEV)
+    key_d = qkv_d[:, 128:128 + D].contiguous().view(N, Hkv, Dh)
+    value_d = qkv_d[:, 128 + 2 * D:].view(N, Hkv, Dh)
+    kc_d, vc_d = kc.to(DEV), vc.to(DEV)
+    ops.store_kvcache(key_d, value_d, kc_d, vc_d, slots.to(DEV))
+    assert torch.equal(kc_d.cpu().view(torch.int16), kc_ref.view(torch.int16))
+    assert torch.equal(vc_d.cpu().view(torch.int16), vc_ref.view(torch.int16))
+
+
+def test_store_kvcache_empty_and_out_of_range(ops):
+    kc = torch.zeros(2, 16, 1, 8, dtype=BF, device=DEV)
+    vc = torch.zeros_like(kc)
+    key = torch.ones(2, 1, 8, dtype=BF, device=DEV)
+    ops.store_kvcache(key[:0], key[:0], kc, vc, torch.zeros(0, dtype=torch.int32, device=DEV))
+    ops.store_kvcache(key, key, kc, vc, torch.tensor([5, 32], dtype=torch.int32, device=DEV))  # 32 == num_slots
+    assert kc.float().sum().item() == 8.0 and kc.view(-1, 8)[5].float().sum().item() == 8.0
+
+
+def test_store_kvcache_fp8_bit_exact(ops):
+    N, Hkv, Dh, nblk, bs = 200, 8, 128, 2, 256
+    key = (torch.randn(N, Hkv, Dh, generator=g(1)) * 2).to(BF)
+    value = (torch.randn(N, Hkv, Dh, generator=g(2)) * 2).to(BF)
+    key[0, 0, 0] = 1000.0; value[1, 1, 1] = -1000.0               # saturation
+    ks = torch.rand(Hkv, generator=g(3)) * 0.02 + 0.005
+    vs = torch.rand(Hkv, generator=g(4)) * 0.02 + 0.005
+    slots = torch.randperm(nblk * bs, generator=g(5))[:N].to(torch.int32)
+    kc = torch.zeros(nblk, bs, Hkv, Dh, dtype=torch.float8_e4m3fn)
+    vc = torch.zeros_like(kc)
+    O.store_kvcache_fp8(key, value, kc, vc, slots, ks, vs)
+    kc_d, vc_d = torch.zeros_like(kc, device=DEV), torch.zeros_like(vc, device=DEV)
+    ops.store_kvcache(key.to(DEV), value.to(DEV), kc_d, vc_d, slots.to(DEV), ks.to(DEV), vs.to(DEV))
+    assert torch.equal(kc_d.cpu().view(torch.uint8), kc.view(torch.uint8))
+    assert torch.equal(vc_d.cpu().view(torch.uint8), vc.view(torch.uint8))
+
+
+# ----------------------------------------------------------------------------- a5 / a6
+@pytest.mark.parametrize("rows,cols", [(1, 1024), (5, 128), (33, 4096), (7, 5120), (3, 12288), (2, 16384), (300, 1024)])
+def test_rmsnorm(ops, rows, cols):
+    x = (torch.randn(rows, cols, generator=g(rows)) * 2).to(BF)
+    w = (1 + 0.2 * torch.randn(cols, generator=g(cols))).to(BF)
+    ref = O.rms_norm(x, w, 1e-6)
+    got = ops.rms_norm(x.to(DEV), w.to(DEV), 1e-6)
+    assert_close_bf16(got, ref)
+
+
+def test_rmsnorm_per_head_strided_view(ops):
+    N, Hq, Hkv, Dh = 19, 16, 8, 128
+    qkv = torch.randn(N, (Hq + 2 * Hkv) * Dh, generator=g(3)).to(BF)
+    w = (1 + 0.2 * torch.randn(Dh, generator=g(4))).to(BF)
+    q = qkv[:, :Hq * Dh].view(N, Hq, Dh)
+    k = qkv[:, Hq * Dh:(Hq + Hkv) * Dh].view(N, Hkv, Dh)
+    qd = qkv.to(DEV)
+    got_q = ops.rms_norm(qd[:, :Hq * Dh].view(N, Hq, Dh), w.to(DEV), 1e-6)
+    got_k = ops.rms_norm(qd[:, Hq * Dh:(Hq + Hkv) * Dh].view(N, Hkv, Dh), w.to(DEV), 1e-6)
+    assert got_q.is_contiguous() and got_q.shape == (N, Hq, Dh)
+    assert_close_bf16(got_q, O.rms_norm(q, w, 1e-6))
+    assert_close_bf16(got_k, O.rms_norm(k, w, 1e-6))
+
+
+@pytest.mark.parametrize("rows,cols", [(1, 1024), (4, 1024), (64, 4096), (9, 5120), (513, 1024)])
+def test_add_rmsnorm(ops, rows, cols):
+    x = torch.randn(rows, cols, generator=g(rows + 1)).to(BF)
+    r = (torch.randn(rows, cols, generator=g(rows + 2)) * 3).to(BF)
+    w = (1 + 0.2 * torch.randn(cols, generator=g(cols))).to(BF)
+    y_ref, r_ref = O.add_rms_norm(x, r, w, 1e-6)
+    y, ro = ops.add_rms_norm(x.to(DEV), r.to(DEV), w.to(DEV), 1e-6)
+    assert torch.equal(ro.cpu().view(torch.int16), r_ref.view(torch.int16))       # one exact fp32 add + one rounding
+    assert_close_bf16(y, y_ref)
+
+
+# ----------------------------------------------------------------------------- a7
+@pytest.mark.parametrize("N,Hq,Hkv", [(1, 16, 8), (37, 32, 8), (512, 16, 8), (5, 64, 8)])
+def test_rope_bit_exact(ops, N, Hq, Hkv):
+    Dh, maxpos = 128, 4096
+    tab = O.rope_table(Dh, maxpos, 1e6)
+    pos = torch.randint(0, maxpos, (N,), generator=g(N))
+    pos[0] = 0
+    qkv = torch.randn(N, (Hq + 2 * Hkv) * Dh, generator=g(N + 1)).to(BF)
+    q, k = qkv[:, :Hq * Dh], qkv[:, Hq * Dh:(Hq + Hkv) * Dh]            # strided rows
+    q_ref, k_ref = O.rope(pos, q, k, tab, Dh)
+    qd = qkv.to(DEV)
+    qg, kg = ops.rope(pos.to(DEV), qd[:, :Hq * Dh], qd[:, Hq * Dh:(Hq + Hkv) * Dh], tab.to(DEV), Dh)
+    # products and sums are rounded separately in fp32, the table comes from the host: bit-exact
+    assert torch.equal(qg.cpu().view(torch.int16), q_ref.view(torch.int16))
+    assert torch.equal(kg.cpu().view(torch.int16), k_ref.view(torch.int16))
+
+
+# ----------------------------------------------------------------------------- fused q/k-norm + rope + store
+@pytest.mark.parametrize("N,Hq,Hkv,want_kv", [(1, 16, 8, False), (45, 32, 8, True), (600, 16, 8, True), (3, 64, 8, False)])
+def test_qknorm_rope_store_equals_unfused_sequence(ops, N, Hq, Hkv, want_kv):
+    Dh, maxpos, nblk, bs = 128, 2048, 4, 256
+    tab = O.rope_table(Dh, maxpos, 1e6)
+    pos = torch.randint(0, maxpos, (N,), generator=g(N))
+    qkv = torch.randn(N, (Hq + 2 * Hkv) * Dh, generator=g(N + 1)).to(BF)
+    qw = (1 + 0.2 * torch.randn(Dh, generator=g(7))).to(BF)
+    kw = (1 + 0.2 * torch.randn(Dh, generator=g(8))).to(BF)
+    slots = torch.randperm(nblk * bs, generator=g(9))[:N].to(torch.int32)
+    if N > 2:
+        slots[1] = -1
+    q, k, v = qkv.split([Hq * Dh, Hkv * Dh, Hkv * Dh], dim=-1)
+    qn = O.rms_norm(q.view(N, Hq, Dh), qw, 1e-6).view(N, -1)
+    kn = O.rms_norm(k.view(N, Hkv, Dh), kw, 1e-6).view(N, -1)
+    q_ref, k_ref = O.rope(pos, qn, kn, tab, Dh)
+    kc = torch.randn(nblk, bs, Hkv, Dh, generator=g(10)).to(BF)
+    vc = torch.randn(nblk, bs, Hkv, Dh, generator=g(11)).to(BF)
+    kc_ref, vc_ref = kc.clone(), vc.clone()
+    O.store_kvcache(k_ref.view(N, Hkv, Dh), v.view(N, Hkv, Dh), kc_ref, vc_ref, slots)
+    kc_d, vc_d = kc.to(DEV), vc.to(DEV)
+    qg, kg, vg = ops.qknorm_rope_store(qkv.to(DEV), qw.to(DEV), kw.to(DEV), 1e-6, pos.to(DEV), tab.to(DEV),
+                                       Hq, Hkv, Dh, kc_d, vc_d, slots.to(DEV), want_kv=want_kv)
+    assert_close_bf16(qg, q_ref, max_ulp=1.0, min_exact=0.99)
+    if want_kv:
+        assert_close_bf16(kg, k_ref, max_ulp=1.0, min_exact=0.99)
+        assert torch.equal(vg.cpu().view(torch.int16), v.contiguous().view(torch.int16))
+    assert torch.equal(vc_d.cpu().view(torch.int16), vc_ref.view(torch.int16))        # V rows are a bit copy
+    assert_close_bf16(kc_d, kc_ref, max_ulp=1.0, min_exact=0.99)
+    # the cache holds exactly what the kernel returned for K, and untouched rows are untouched
+    if want_kv:
+        flat = kc_d.view(-1, Hkv * Dh)
+        for i in range(0, N, max(1, N // 7)):
+            if slots[i] >= 0:
+                assert torch.equal(flat[slots[i].item()], kg[i])
+    untouched = torch.ones(nblk * bs, dtype=torch.bool); untouched[slots[slots >= 0].long()] = False
+    assert torch.equal(kc_d.cpu().view(-1, Hkv * Dh)[untouched], kc.view(-1, Hkv * Dh)[untouched])
+
+
+# ----------------------------------------------------------------------------- a8
+@pytest.mark.parametrize("rows,inter", [(1, 3072), (4, 3072), (130, 12288), (7, 25600)])
+def test_silu_and_mul(ops, rows, inter):
+    x = (torch.randn(rows, 2 * inter, generator=g(rows)) * 3).to(BF)
+    assert_close_bf16(ops.silu_and_mul(x.to(DEV)), O.silu_and_mul(x), max_ulp=1.0, min_exact=0.999)
+
+
+# ----------------------------------------------------------------------------- a9
+@pytest.mark.parametrize("rows,vocab", [(1, 151936), (4, 151936), (256, 151936), (3, 1000), (2, 8), (5, 4099)])
+def test_argmax_bit_exact(ops, rows, vocab):
+    pad = (-vocab) % 8
+    buf = torch.randn(rows, vocab + pad, generator=g(rows + vocab)).to(BF)
+    logits = buf[:, :vocab]
+    if vocab > 100:                                                # plant ties: first index must win
+        logits[0, 77] = 9.0; logits[0, 50] = 9.0; logits[0, vocab - 1] = 9.0
+    ref = O.greedy_sample(logits)
+    got = ops.argmax(buf.to(DEV)[:, :vocab])
+    assert got.dtype == torch.int64
+    assert torch.equal(got.cpu(), ref)
+
+
+def test_argmax_all_negative_and_zero_signs(ops):
+    l = torch.full((2, 64), -5.0).to(BF)
+    l[0, 40] = -0.0; l[0, 41] = 0.0
+    l[1, 63] = -4.0
+    assert ops.argmax(l.to(DEV)).tolist() == O.greedy_sample(l).tolist() == [40, 63]
+
+
+# ----------------------------------------------------------------------------- K9
+def test_embedding_bit_exact(ops):
+    w = torch.randn(1000, 1024, generator=g(0)).to(BF)
+    ids = torch.randint(0, 1000, (77,), generator=g(1))
+    got = ops.embedding(ids.to(DEV), w.to(DEV))
+    assert torch.equal(got.cpu().view(torch.int16), O.embedding(ids, w).view(torch.int16))

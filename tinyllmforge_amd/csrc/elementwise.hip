@@ -1,0 +1,504 @@
+// Single-pass, 128-bit vectorised elementwise / row-reduction kernels:
+// RMSNorm (+ residual), RoPE, SiLU-and-mul, embedding gather, greedy argmax.
+// All are HBM bound; each element is read once and written once.
+#include "common.h"
+
+namespace tlf {
+
+// --------------------------------------------------------------------------
+// RMSNorm / add-RMSNorm (reference: tinyvllm/layers/layernorm.py:21-45).
+// TPR threads share one row, each holding up to MAXC chunks of 8 elements in
+// registers, so x is read once.  Rounding points follow the reference:
+//   n = bf16(s * rsqrt(mean(s^2) + eps));  y = bf16(float(n) * float(w)).
+template <int TPR, int MAXC, bool ADD>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(
+    const unsigned short *__restrict__ x, int64_t x_outer_stride,
+    const unsigned short *__restrict__ residual, const unsigned short *__restrict__ weight,
+    unsigned short *__restrict__ y, unsigned short *__restrict__ residual_out, int64_t rows,
+    int32_t inner, int32_t cols, float eps) {
+  constexpr int kRowsPerBlock = 256 / TPR;
+  const int tid = threadIdx.x;
+  const int sub = tid % TPR;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + tid / TPR;
+  const bool active = row < rows;
+  const int nchunks = cols / 8;
+  const int64_t safe_row = active ? row : 0;
+  const unsigned short *xr = x + (safe_row / inner) * x_outer_stride + (safe_row % inner) * cols;
+  const int64_t out_off = safe_row * cols;
+
+  float v[MAXC][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int chunk = sub + c * TPR;
+    if (active && chunk < nchunks) {
+      uint4 p = *reinterpret_cast<const uint4 *>(xr + chunk * 8);
+      unpack8(p, v[c]);
+      if (ADD) {
+        float r[8];
+        uint4 pr = *reinterpret_cast<const uint4 *>(residual + out_off + chunk * 8);
+        unpack8(pr, r);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[c][i] = __fadd_rn(v[c][i], r[i]);
+        *reinterpret_cast<uint4 *>(residual_out + out_off + chunk * 8) = pack8(v[c]);
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss = fmaf(v[c][i], v[c][i], ss);
+    }
+  }
+  // reduce over the TPR threads of the row
+  if (TPR <= 64) {
+#pragma unroll
+    for (int o = TPR / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+  } else {
+    __shared__ float part[256 / 64];
+    ss = wave_sum(ss);
+    if ((tid & 63) == 0) part[tid >> 6] = ss;
+    __syncthreads();
+    ss = 0.f;
+#pragma unroll
+    for (int w = 0; w < TPR / 64; ++w) ss += part[w];
+  }
+  const float var = ss / static_cast<float>(cols);
+  const float inv = 1.0f / sqrtf(var + eps);
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int chunk = sub + c * TPR;
+    if (active && chunk < nchunks) {
+      float w[8];
+      uint4 pw = *reinterpret_cast<const uint4 *>(weight + chunk * 8);
+      unpack8(pw, w);
+      float o[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float n = bf16_bits_to_float(float_to_bf16_bits(__fmul_rn(v[c][i], inv)));
+        o[i] = __fmul_rn(n, w[i]);
+      }
+      *reinterpret_cast<uint4 *>(y + out_off + chunk * 8) = pack8(o);
+    }
+  }
+}
+
+template <bool ADD>
+int launch_rmsnorm(const void *x, int64_t x_outer_stride, const void *residual, const void *weight,
+                   void *y, void *residual_out, int64_t rows, int32_t inner, int32_t cols,
+                   float eps, hipStream_t stream) {
+  auto xs = static_cast<const unsigned short *>(x);
+  auto rs = static_cast<const unsigned short *>(residual);
+  auto ws = static_cast<const unsigned short *>(weight);
+  auto ys = static_cast<unsigned short *>(y);
+  auto ro = static_cast<unsigned short *>(residual_out);
+#define TLF_RMS(TPR, MAXC)                                                                       \
+  hipLaunchKernelGGL((rmsnorm_kernel<TPR, MAXC, ADD>),                                            \
+                     dim3(static_cast<unsigned>((rows + (256 / TPR) - 1) / (256 / TPR))),         \
+                     dim3(256), 0, stream, xs, x_outer_stride, rs, ws, ys, ro, rows, inner, cols, \
+                     eps)
+  if (cols <= 128) TLF_RMS(16, 1);
+  else if (cols <= 512) TLF_RMS(64, 1);
+  else if (cols <= 2048) TLF_RMS(64, 4);
+  else if (cols <= 8192) TLF_RMS(256, 4);
+  else TLF_RMS(256, 8);
+#undef TLF_RMS
+  return launch_status();
+}
+
+// --------------------------------------------------------------------------
+// RoPE (reference: tinyvllm/layers/rotary_embedding.py:5-15, 41-57).
+// One thread rotates 8 pairs (i, i + head_dim/2) of one head of one token.
+__global__ __launch_bounds__(256) void rope_kernel(
+    const int64_t *__restrict__ positions, const unsigned short *__restrict__ q, int64_t q_stride,
+    const unsigned short *__restrict__ k, int64_t k_stride, const float *__restrict__ cos_sin,
+    unsigned short *__restrict__ q_out, unsigned short *__restrict__ k_out, int32_t n,
+    int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int32_t max_pos) {
+  const int half = head_dim / 2;
+  const int cpt = half / 8;  // chunks per head
+  const int heads = num_q_heads + num_kv_heads;
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t total = static_cast<int64_t>(n) * heads * cpt;
+  if (item >= total) return;
+  const int c = static_cast<int>(item % cpt);
+  const int h = static_cast<int>((item / cpt) % heads);
+  const int64_t tok = item / (static_cast<int64_t>(cpt) * heads);
+  const int64_t pos = positions[tok];
+  if (pos < 0 || pos >= max_pos) return;
+  const bool is_q = h < num_q_heads;
+  const int hh = is_q ? h : h - num_q_heads;
+  const unsigned short *src = (is_q ? q + tok * q_stride : k + tok * k_stride) + hh * head_dim;
+  unsigned short *dst = (is_q ? q_out + tok * static_cast<int64_t>(num_q_heads) * head_dim
+                              : k_out + tok * static_cast<int64_t>(num_kv_heads) * head_dim) +
+                        hh * head_dim;
+  float x1[8], x2[8];
+  unpack8(*reinterpret_cast<const uint4 *>(src + c * 8), x1);
+  unpack8(*reinterpret_cast<const uint4 *>(src + half + c * 8), x2);
+  const float *cs = cos_sin + pos * head_dim;
+  float y1[8], y2[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float co = cs[c * 8 + i];
+    const float si = cs[half + c * 8 + i];
+    y1[i] = __fsub_rn(__fmul_rn(co, x1[i]), __fmul_rn(si, x2[i]));
+    y2[i] = __fadd_rn(__fmul_rn(co, x2[i]), __fmul_rn(si, x1[i]));
+  }
+  *reinterpret_cast<uint4 *>(dst + c * 8) = pack8(y1);
+  *reinterpret_cast<uint4 *>(dst + half + c * 8) = pack8(y2);
+}
+
+// --------------------------------------------------------------------------
+// Fused q/k RMSNorm + RoPE + KV-cache store over the qkv projection
+// (reference op sequence: tinyvllm/models/qwen3.py:79-94, layers/attention.py:94-95).
+// 16 lanes own one head (8 dims each); lanes j < 8 hold the first half of the
+// head, lanes j >= 8 the second, so the RoPE partner of lane j is lane j ^ 8.
+__global__ __launch_bounds__(256) void qknorm_rope_store_kernel(
+    const unsigned short *__restrict__ qkv, int64_t qkv_stride,
+    const unsigned short *__restrict__ qw, const unsigned short *__restrict__ kw, float eps,
+    const int64_t *__restrict__ positions, const float *__restrict__ cos_sin, int32_t max_pos,
+    unsigned short *__restrict__ q_out, unsigned short *__restrict__ k_out,
+    unsigned short *__restrict__ v_out, unsigned char *__restrict__ k_cache,
+    unsigned char *__restrict__ v_cache, const int32_t *__restrict__ slot_mapping,
+    int64_t num_slots, int32_t kv_dtype, const float *__restrict__ k_scale,
+    const float *__restrict__ v_scale, int32_t num_q_heads, int32_t num_kv_heads) {
+  constexpr int kDh = 128;
+  const int64_t tok = blockIdx.x;
+  const int head = blockIdx.y * 16 + threadIdx.x / 16;
+  const int j = threadIdx.x % 16;
+  const int heads = num_q_heads + 2 * num_kv_heads;
+  if (head >= heads) return;  // whole 16-lane groups leave together
+  const unsigned short *src = qkv + tok * qkv_stride + head * kDh + j * 8;
+  const uint4 raw = *reinterpret_cast<const uint4 *>(src);
+  const bool is_q = head < num_q_heads;
+  const bool is_k = !is_q && head < num_q_heads + num_kv_heads;
+  const int kvh = is_q ? 0 : (is_k ? head - num_q_heads : head - num_q_heads - num_kv_heads);
+  int64_t slot = -1;
+  if (!is_q && slot_mapping != nullptr) {
+    slot = slot_mapping[tok];
+    if (slot >= num_slots) slot = -1;
+  }
+  uint4 outp = raw;
+  if (is_q || is_k) {
+    float v[8];
+    unpack8(raw, v);
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) ss = fmaf(v[i], v[i], ss);
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    const float inv = 1.0f / sqrtf(ss / static_cast<float>(kDh) + eps);
+    float w[8];
+    unpack8(*reinterpret_cast<const uint4 *>((is_q ? qw : kw) + j * 8), w);
+    float nrm[8], other[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float nn = bf16_bits_to_float(float_to_bf16_bits(__fmul_rn(v[i], inv)));
+      nrm[i] = bf16_bits_to_float(float_to_bf16_bits(__fmul_rn(nn, w[i])));
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) other[i] = __shfl_xor(nrm[i], 8, 64);
+    const int64_t pos = positions[tok];
+    const bool pos_ok = pos >= 0 && pos < max_pos;
+    const float *cs = cos_sin + (pos_ok ? pos : 0) * kDh;
+    const int cj = (j % 8) * 8;
+    float o[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float co = cs[cj + i];
+      const float si = cs[64 + cj + i];
+      // lanes j < 8: cos*x1 - sin*x2 ; lanes j >= 8: cos*x2 + sin*x1
+      const float a = __fmul_rn(co, nrm[i]);
+      const float b = __fmul_rn(si, other[i]);
+      o[i] = (j < 8) ? __fsub_rn(a, b) : __fadd_rn(a, b);
+      if (!pos_ok) o[i] = nrm[i];
+    }
+    outp = pack8(o);
+  }
+  if (is_q) {
+    *reinterpret_cast<uint4 *>(q_out + tok * static_cast<int64_t>(num_q_heads) * kDh + head * kDh +
+                               j * 8) = outp;
+    return;
+  }
+  const int64_t row_elems = static_cast<int64_t>(num_kv_heads) * kDh;
+  unsigned short *lin = is_k ? k_out : v_out;
+  if (lin != nullptr) *reinterpret_cast<uint4 *>(lin + tok * row_elems + kvh * kDh + j * 8) = outp;
+  if (slot < 0) return;
+  unsigned char *cache = is_k ? k_cache : v_cache;
+  if (kv_dtype == TLF_KV_BF16) {
+    *reinterpret_cast<uint4 *>(cache + (slot * row_elems + kvh * kDh + j * 8) * 2) = outp;
+  } else {
+    float f[8];
+    unpack8(outp, f);
+    const float s = (is_k ? k_scale : v_scale)[kvh];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = fminf(fmaxf(f[i] / s, -448.0f), 448.0f);
+    int lo = 0, hi = 0;
+    lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], lo, false);
+    lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
+    hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], hi, false);
+    hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
+    *reinterpret_cast<int2 *>(cache + slot * row_elems + kvh * kDh + j * 8) = make_int2(lo, hi);
+  }
+}
+
+// --------------------------------------------------------------------------
+// SiLU-and-mul (reference: tinyvllm/layers/activation.py:11-14, eager rounding).
+__global__ __launch_bounds__(256) void silu_and_mul_kernel(const unsigned short *__restrict__ x,
+                                                           unsigned short *__restrict__ y,
+                                                           int64_t rows, int32_t inter) {
+  const int cpr = inter / 8;
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (item >= rows * cpr) return;
+  const int64_t r = item / cpr;
+  const int c = static_cast<int>(item % cpr);
+  const unsigned short *xr = x + r * 2 * inter;
+  float g[8], u[8], o[8];
+  unpack8(*reinterpret_cast<const uint4 *>(xr + c * 8), g);
+  unpack8(*reinterpret_cast<const uint4 *>(xr + inter + c * 8), u);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float s = g[i] / (1.0f + expf(-g[i]));
+    o[i] = __fmul_rn(bf16_bits_to_float(float_to_bf16_bits(s)), u[i]);
+  }
+  *reinterpret_cast<uint4 *>(y + r * inter + c * 8) = pack8(o);
+}
+
+// --------------------------------------------------------------------------
+// Embedding gather (reference: tinyvllm/layers/embed_head.py:38).
+__global__ __launch_bounds__(256) void embedding_kernel(const int64_t *__restrict__ ids,
+                                                        const unsigned short *__restrict__ weight,
+                                                        unsigned short *__restrict__ y,
+                                                        int32_t vocab, int32_t cols) {
+  const int64_t tok = blockIdx.x;
+  const int64_t id = ids[tok];
+  const bool ok = id >= 0 && id < vocab;
+  const unsigned short *src = weight + (ok ? id : 0) * cols;
+  unsigned short *dst = y + tok * cols;
+  for (int c = threadIdx.x * 8; c < cols; c += blockDim.x * 8) {
+    uint4 p = make_uint4(0, 0, 0, 0);
+    if (ok) p = *reinterpret_cast<const uint4 *>(src + c);
+    *reinterpret_cast<uint4 *>(dst + c) = p;
+  }
+}
+
+// --------------------------------------------------------------------------
+// Greedy argmax (reference: tinyvllm/layers/sampler.py:13-14,21).
+// key = (order-preserving image of the bf16 value) << 32 | (~index): the maximum
+// key is the largest value with the smallest index among ties.
+constexpr int kArgmaxMaxChunks = 128;
+
+__device__ __forceinline__ unsigned long long argmax_key(unsigned short bits, unsigned int idx) {
+  if (bits == 0x8000u) bits = 0;  // -0 == +0
+  const unsigned int ord = (bits & 0x8000u) ? (~bits & 0xffffu) : (bits | 0x8000u);
+  return (static_cast<unsigned long long>(ord) << 32) | (0xffffffffu - idx);
+}
+
+__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    unsigned int lo = __shfl_xor(static_cast<unsigned int>(v), o, 64);
+    unsigned int hi = __shfl_xor(static_cast<unsigned int>(v >> 32), o, 64);
+    unsigned long long other = (static_cast<unsigned long long>(hi) << 32) | lo;
+    v = other > v ? other : v;
+  }
+  return v;
+}
+
+__global__ __launch_bounds__(256) void argmax_partial_kernel(
+    const unsigned short *__restrict__ logits, int64_t row_stride, int32_t vocab,
+    unsigned long long *__restrict__ partial, int32_t nchunks) {
+  const int row = blockIdx.y;
+  const int chunk = blockIdx.x;
+  const unsigned short *lr = logits + row * row_stride;
+  const int nvec = vocab / 8;
+  const int vec_per_chunk = (nvec + nchunks - 1) / nchunks;
+  const int v0 = chunk * vec_per_chunk;
+  const int v1 = min(v0 + vec_per_chunk, nvec);
+  unsigned long long best = 0;
+  for (int v = v0 + threadIdx.x; v < v1; v += blockDim.x) {
+    Pack16 p;
+    p.u = *reinterpret_cast<const uint4 *>(lr + static_cast<int64_t>(v) * 8);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const unsigned long long key = argmax_key(p.s[i], static_cast<unsigned int>(v * 8 + i));
+      best = key > best ? key : best;
+    }
+  }
+  if (chunk == 0) {  // scalar tail when vocab is not a multiple of 8
+    const int t = nvec * 8 + threadIdx.x;
+    if (t < vocab) {
+      const unsigned long long key = argmax_key(lr[t], static_cast<unsigned int>(t));
+      best = key > best ? key : best;
+    }
+  }
+  __shared__ unsigned long long part[4];
+  best = wave_max_u64(best);
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = best;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w) best = part[w] > best ? part[w] : best;
+    partial[static_cast<int64_t>(row) * nchunks + chunk] = best;
+  }
+}
+
+__global__ __launch_bounds__(64) void argmax_final_kernel(
+    const unsigned long long *__restrict__ partial, int32_t nchunks, int64_t *__restrict__ out) {
+  const int row = blockIdx.x;
+  unsigned long long best = 0;
+  for (int c = threadIdx.x; c < nchunks; c += 64) {
+    const unsigned long long k = partial[static_cast<int64_t>(row) * nchunks + c];
+    best = k > best ? k : best;
+  }
+  best = wave_max_u64(best);
+  if (threadIdx.x == 0) out[row] = static_cast<int64_t>(0xffffffffu - static_cast<unsigned int>(best));
+}
+
+inline int argmax_chunks(int32_t rows, int32_t vocab) {
+  int by_rows = (1024 + rows - 1) / rows;
+  int by_vocab = (vocab + 2047) / 2048;
+  int n = by_rows < by_vocab ? by_rows : by_vocab;
+  if (n < 1) n = 1;
+  if (n > kArgmaxMaxChunks) n = kArgmaxMaxChunks;
+  return n;
+}
+
+}  // namespace tlf
+
+// ============================================================================ C ABI
+using namespace tlf;
+
+extern "C" int tlf_rmsnorm(const void *x, int64_t x_outer_stride, const void *weight, void *y,
+                           int32_t outer, int32_t inner, int32_t cols, float eps, void *stream) {
+  if (outer == 0 || inner == 0) return TLF_OK;
+  if (!x || !weight || !y) return TLF_E_NULL;
+  if (outer < 0 || inner < 0 || cols <= 0 || cols % 8 || cols > 16384) return TLF_E_SHAPE;
+  if (x_outer_stride < static_cast<int64_t>(inner) * cols) return TLF_E_SHAPE;
+  if (!aligned16(x) || !aligned16(weight) || !aligned16(y) || x_outer_stride % 8) return TLF_E_ALIGN;
+  return launch_rmsnorm<false>(x, x_outer_stride, nullptr, weight, y, nullptr,
+                               static_cast<int64_t>(outer) * inner, inner, cols, eps,
+                               static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tlf_add_rmsnorm(const void *x, const void *residual, const void *weight, void *y,
+                               void *residual_out, int32_t rows, int32_t cols, float eps,
+                               void *stream) {
+  if (rows == 0) return TLF_OK;
+  if (!x || !residual || !weight || !y || !residual_out) return TLF_E_NULL;
+  if (rows < 0 || cols <= 0 || cols % 8 || cols > 16384) return TLF_E_SHAPE;
+  if (!aligned16(x) || !aligned16(residual) || !aligned16(weight) || !aligned16(y) ||
+      !aligned16(residual_out))
+    return TLF_E_ALIGN;
+  return launch_rmsnorm<true>(x, cols, residual, weight, y, residual_out, rows, 1, cols, eps,
+                              static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tlf_rope(const int64_t *positions, const void *q, int64_t q_stride, const void *k,
+                        int64_t k_stride, const float *cos_sin, void *q_out, void *k_out,
+                        int32_t n, int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                        int32_t max_pos, void *stream) {
+  if (n == 0) return TLF_OK;
+  if (!positions || !q || !k || !cos_sin || !q_out || !k_out) return TLF_E_NULL;
+  if (n < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || head_dim <= 0 || head_dim % 16 ||
+      max_pos <= 0)
+    return TLF_E_SHAPE;
+  if (q_stride < static_cast<int64_t>(num_q_heads) * head_dim ||
+      k_stride < static_cast<int64_t>(num_kv_heads) * head_dim)
+    return TLF_E_SHAPE;
+  if (!aligned16(q) || !aligned16(k) || !aligned16(q_out) || !aligned16(k_out) || q_stride % 8 ||
+      k_stride % 8)
+    return TLF_E_ALIGN;
+  const int64_t total = static_cast<int64_t>(n) * (num_q_heads + num_kv_heads) * (head_dim / 16);
+  hipLaunchKernelGGL(rope_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), positions,
+                     static_cast<const unsigned short *>(q), q_stride,
+                     static_cast<const unsigned short *>(k), k_stride, cos_sin,
+                     static_cast<unsigned short *>(q_out), static_cast<unsigned short *>(k_out), n,
+                     num_q_heads, num_kv_heads, head_dim, max_pos);
+  return launch_status();
+}
+
+extern "C" int tlf_qknorm_rope_store(const void *qkv, int64_t qkv_stride, const void *q_norm_weight,
+                                     const void *k_norm_weight, float eps, const int64_t *positions,
+                                     const float *cos_sin, int32_t max_pos, void *q_out,
+                                     void *k_out, void *v_out, void *k_cache, void *v_cache,
+                                     const int32_t *slot_mapping, int64_t num_slots,
+                                     int32_t kv_dtype, const float *k_scale, const float *v_scale,
+                                     int32_t n, int32_t num_q_heads, int32_t num_kv_heads,
+                                     int32_t head_dim, void *stream) {
+  if (n == 0) return TLF_OK;
+  if (!qkv || !q_norm_weight || !k_norm_weight || !positions || !cos_sin || !q_out)
+    return TLF_E_NULL;
+  if (head_dim != 128) return TLF_E_UNSUPPORTED;
+  if (n < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || max_pos <= 0) return TLF_E_SHAPE;
+  const int heads = num_q_heads + 2 * num_kv_heads;
+  if (qkv_stride < static_cast<int64_t>(heads) * head_dim) return TLF_E_SHAPE;
+  if (slot_mapping != nullptr) {
+    if (!k_cache || !v_cache) return TLF_E_NULL;
+    if (num_slots <= 0) return TLF_E_SHAPE;
+    if (kv_dtype == TLF_KV_FP8_E4M3) {
+      if (!k_scale || !v_scale) return TLF_E_NULL;
+    } else if (kv_dtype != TLF_KV_BF16) {
+      return TLF_E_UNSUPPORTED;
+    }
+    if (!aligned16(k_cache) || !aligned16(v_cache)) return TLF_E_ALIGN;
+  }
+  if (!aligned16(qkv) || qkv_stride % 8 || !aligned16(q_out) || !aligned16(q_norm_weight) ||
+      !aligned16(k_norm_weight) || (k_out && !aligned16(k_out)) || (v_out && !aligned16(v_out)))
+    return TLF_E_ALIGN;
+  hipLaunchKernelGGL(qknorm_rope_store_kernel, dim3(n, (heads + 15) / 16), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const unsigned short *>(qkv),
+                     qkv_stride, static_cast<const unsigned short *>(q_norm_weight),
+                     static_cast<const unsigned short *>(k_norm_weight), eps, positions, cos_sin,
+                     max_pos, static_cast<unsigned short *>(q_out),
+                     static_cast<unsigned short *>(k_out), static_cast<unsigned short *>(v_out),
+                     static_cast<unsigned char *>(k_cache), static_cast<unsigned char *>(v_cache),
+                     slot_mapping, num_slots, kv_dtype, k_scale, v_scale, num_q_heads,
+                     num_kv_heads);
+  return launch_status();
+}
+
+extern "C" int tlf_silu_and_mul(const void *x, void *y, int32_t rows, int32_t inter, void *stream) {
+  if (rows == 0) return TLF_OK;
+  if (!x || !y) return TLF_E_NULL;
+  if (rows < 0 || inter <= 0 || inter % 8) return TLF_E_SHAPE;
+  if (!aligned16(x) || !aligned16(y)) return TLF_E_ALIGN;
+  const int64_t total = static_cast<int64_t>(rows) * (inter / 8);
+  hipLaunchKernelGGL(silu_and_mul_kernel, dim3(static_cast<unsigned>((total + 255) / 256)),
+                     dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const unsigned short *>(x), static_cast<unsigned short *>(y),
+                     static_cast<int64_t>(rows), inter);
+  return launch_status();
+}
+
+extern "C" int tlf_embedding(const int64_t *ids, const void *weight, void *y, int32_t n,
+                             int32_t vocab, int32_t cols, void *stream) {
+  if (n == 0) return TLF_OK;
+  if (!ids || !weight || !y) return TLF_E_NULL;
+  if (n < 0 || vocab <= 0 || cols <= 0 || cols % 8) return TLF_E_SHAPE;
+  if (!aligned16(weight) || !aligned16(y)) return TLF_E_ALIGN;
+  hipLaunchKernelGGL(embedding_kernel, dim3(n), dim3(256), 0, static_cast<hipStream_t>(stream), ids,
+                     static_cast<const unsigned short *>(weight), static_cast<unsigned short *>(y),
+                     vocab, cols);
+  return launch_status();
+}
+
+extern "C" size_t tlf_argmax_workspace_bytes(int32_t rows, int32_t vocab) {
+  (void)vocab;
+  if (rows <= 0) return 0;
+  return static_cast<size_t>(rows) * kArgmaxMaxChunks * sizeof(unsigned long long);
+}
+
+extern "C" int tlf_argmax(const void *logits, int64_t row_stride, int64_t *out, int32_t rows,
+                          int32_t vocab, void *workspace, size_t workspace_bytes, void *stream) {
+  if (rows == 0) return TLF_OK;
+  if (!logits || !out) return TLF_E_NULL;
+  if (rows < 0 || vocab <= 0 || row_stride < vocab) return TLF_E_SHAPE;
+  if (!aligned16(logits) || row_stride % 8) return TLF_E_ALIGN;
+  if (!workspace || workspace_bytes < tlf_argmax_workspace_bytes(rows, vocab) ||
+      (reinterpret_cast<uintptr_t>(workspace) & 7u))
+    return TLF_E_WORKSPACE;
+  const int nchunks = argmax_chunks(rows, vocab);
+  auto part = static_cast<unsigned long long *>(workspace);
+  hipLaunchKernelGGL(argmax_partial_kernel, dim3(nchunks, rows), dim3(256), 0,
+                     static_cast<hipStream_t>(stream),
+                     static_cast<const unsigned short *>(logits), row_stride, vocab, part, nchunks);
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(64), 0,
+                     static_cast<hipStream_t>(stream), part, nchunks, out);
+  return launch_status();
+}

@@ -1,0 +1,275 @@
+"""Tensor-level wrappers over the C ABI: one function per hot-path op.
+
+Each wrapper validates what only Python can see (device, dtype), allocates the
+output through torch (the caller owns every buffer, as in the reference) and
+enqueues the kernel on torch's current stream, so calls are capturable by
+``torch.cuda.graph``.  A tensor that is not on the GPU is an error.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+from ._lib import KV_BF16, KV_FP8_E4M3, check
+
+BF16 = torch.bfloat16
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need(t: torch.Tensor, dtype, name: str):
+    if not t.is_cuda:
+        raise _lib.TlfError(f"{name} must be a GPU tensor (the HIP path has no CPU fallback)")
+    if dtype is not None and t.dtype != dtype:
+        raise _lib.TlfError(f"{name} must be {dtype}, got {t.dtype}")
+
+
+_workspaces: dict = {}
+
+
+def _workspace(nbytes: int, device, tag: str) -> torch.Tensor:
+    """Grow-only scratch buffer per (device, tag, stream-capture state is the caller's concern)."""
+    key = (device, tag)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def kv_dtype_code(cache: torch.Tensor) -> int:
+    if cache.dtype == BF16:
+        return KV_BF16
+    if cache.dtype == torch.float8_e4m3fn:
+        return KV_FP8_E4M3
+    raise _lib.TlfError(f"unsupported KV-cache dtype {cache.dtype}")
+
+
+# ------------------------------------------------------------------ a1
+def store_kvcache(key, value, k_cache, v_cache, slot_mapping, k_scale=None, v_scale=None):
+    """``key``/``value`` ``[N, Hkv, Dh]`` (row stride free), caches ``[nblk, bs, Hkv, Dh]``."""
+    lib = _lib.load()
+    _need(key, BF16, "key"); _need(value, BF16, "value")
+    _need(slot_mapping, torch.int32, "slot_mapping")
+    n, h, d = key.shape
+    assert key.stride(-1) == 1 and value.stride(-1) == 1
+    assert key.stride(1) == d and value.stride(1) == d
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
+    assert slot_mapping.numel() == n
+    num_slots = k_cache.numel() // (h * d)
+    if k_cache.dtype == BF16:
+        check(lib.tlf_store_kvcache(key.data_ptr(), key.stride(0) * 2, value.data_ptr(), value.stride(0) * 2,
+                                    k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(),
+                                    n, h * d * 2, num_slots, _stream()), "tlf_store_kvcache")
+    else:
+        _need(k_scale, torch.float32, "k_scale"); _need(v_scale, torch.float32, "v_scale")
+        check(lib.tlf_store_kvcache_fp8(key.data_ptr(), key.stride(0) * 2, value.data_ptr(), value.stride(0) * 2,
+                                        k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(),
+                                        n, h, d, k_scale.data_ptr(), v_scale.data_ptr(), num_slots, _stream()),
+              "tlf_store_kvcache_fp8")
+
+
+# ------------------------------------------------------------------ a5 / a6
+def rms_norm(x, weight, eps):
+    """``x [..., cols]`` bf16; leading dims may be a strided view ``[outer, inner, cols]``."""
+    lib = _lib.load()
+    _need(x, BF16, "x"); _need(weight, BF16, "weight")
+    cols = x.shape[-1]
+    assert x.stride(-1) == 1
+    if x.dim() == 3 and not x.is_contiguous():
+        outer, inner = x.shape[0], x.shape[1]
+        assert x.stride(1) == cols
+        ostride = x.stride(0)
+    else:
+        x = x if x.is_contiguous() else x.contiguous()
+        outer, inner, ostride = x.numel() // cols, 1, cols
+    y = torch.empty(x.shape, dtype=BF16, device=x.device)
+    check(lib.tlf_rmsnorm(x.data_ptr(), ostride, weight.data_ptr(), y.data_ptr(), outer, inner, cols,
+                          float(eps), _stream()), "tlf_rmsnorm")
+    return y
+
+
+def add_rms_norm(x, residual, weight, eps):
+    lib = _lib.load()
+    _need(x, BF16, "x"); _need(residual, BF16, "residual"); _need(weight, BF16, "weight")
+    assert x.is_contiguous() and residual.is_contiguous() and x.shape == residual.shape
+    cols = x.shape[-1]
+    rows = x.numel() // cols
+    y = torch.empty_like(x)
+    r = torch.empty_like(x)
+    check(lib.tlf_add_rmsnorm(x.data_ptr(), residual.data_ptr(), weight.data_ptr(), y.data_ptr(),
+                              r.data_ptr(), rows, cols, float(eps), _stream()), "tlf_add_rmsnorm")
+    return y, r
+
+
+# ------------------------------------------------------------------ a7
+def rope(positions, q, k, cos_sin, head_dim):
+    lib = _lib.load()
+    _need(positions, torch.int64, "positions"); _need(q, BF16, "q"); _need(k, BF16, "k")
+    _need(cos_sin, torch.float32, "cos_sin_cache")
+    n = positions.numel()
+    assert q.stride(-1) == 1 and k.stride(-1) == 1 and q.dim() == 2 and k.dim() == 2
+    hq, hkv = q.shape[1] // head_dim, k.shape[1] // head_dim
+    qo = torch.empty(q.shape, dtype=BF16, device=q.device)
+    ko = torch.empty(k.shape, dtype=BF16, device=k.device)
+    check(lib.tlf_rope(positions.data_ptr(), q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0),
+                       cos_sin.data_ptr(), qo.data_ptr(), ko.data_ptr(), n, hq, hkv, head_dim,
+                       cos_sin.shape[0], _stream()), "tlf_rope")
+    return qo, ko
+
+
+def qknorm_rope_store(qkv, q_weight, k_weight, eps, positions, cos_sin, num_q_heads, num_kv_heads, head_dim,
+                      k_cache=None, v_cache=None, slot_mapping=None, k_scale=None, v_scale=None,
+                      want_kv=False):
+    """Fused q/k-norm + RoPE + KV store.  Returns ``(q, k, v)``; ``k``/``v`` are None unless ``want_kv``."""
+    lib = _lib.load()
+    _need(qkv, BF16, "qkv"); _need(positions, torch.int64, "positions")
+    n = qkv.shape[0]
+    assert qkv.stride(-1) == 1
+    q = torch.empty(n, num_q_heads * head_dim, dtype=BF16, device=qkv.device)
+    k = v = None
+    if want_kv:
+        k = torch.empty(n, num_kv_heads * head_dim, dtype=BF16, device=qkv.device)
+        v = torch.empty(n, num_kv_heads * head_dim, dtype=BF16, device=qkv.device)
+    has_cache = k_cache is not None and k_cache.numel() > 0 and slot_mapping is not None
+    kvd = kv_dtype_code(k_cache) if has_cache else KV_BF16
+    num_slots = (k_cache.numel() // (num_kv_heads * head_dim)) if has_cache else 0
+    check(lib.tlf_qknorm_rope_store(
+        qkv.data_ptr(), qkv.stride(0), q_weight.data_ptr(), k_weight.data_ptr(), float(eps),
+        positions.data_ptr(), cos_sin.data_ptr(), cos_sin.shape[0], q.data_ptr(),
+        k.data_ptr() if k is not None else None, v.data_ptr() if v is not None else None,
+        k_cache.data_ptr() if has_cache else None, v_cache.data_ptr() if has_cache else None,
+        slot_mapping.data_ptr() if has_cache else None, num_slots, kvd,
+        k_scale.data_ptr() if k_scale is not None else None,
+        v_scale.data_ptr() if v_scale is not None else None,
+        n, num_q_heads, num_kv_heads, head_dim, _stream()), "tlf_qknorm_rope_store")
+    return q, k, v
+
+
+# ------------------------------------------------------------------ a8
+def silu_and_mul(x):
+    lib = _lib.load()
+    _need(x, BF16, "x")
+    assert x.is_contiguous() and x.shape[-1] % 2 == 0
+    inter = x.shape[-1] // 2
+    rows = x.numel() // (2 * inter)
+    y = torch.empty(*x.shape[:-1], inter, dtype=BF16, device=x.device)
+    check(lib.tlf_silu_and_mul(x.data_ptr(), y.data_ptr(), rows, inter, _stream()), "tlf_silu_and_mul")
+    return y
+
+
+# ------------------------------------------------------------------ a9
+def argmax(logits):
+    lib = _lib.load()
+    _need(logits, BF16, "logits")
+    assert logits.dim() == 2 and logits.stride(1) == 1
+    rows, vocab = logits.shape
+    out = torch.empty(rows, dtype=torch.int64, device=logits.device)
+    nbytes = lib.tlf_argmax_workspace_bytes(rows, vocab)
+    ws = _workspace(nbytes, logits.device, "argmax")
+    check(lib.tlf_argmax(logits.data_ptr(), logits.stride(0), out.data_ptr(), rows, vocab,
+                         ws.data_ptr(), ws.numel(), _stream()), "tlf_argmax")
+    return out
+
+
+# ------------------------------------------------------------------ K9
+def embedding(ids, weight):
+    lib = _lib.load()
+    _need(ids, torch.int64, "ids"); _need(weight, BF16, "weight")
+    assert weight.is_contiguous() and ids.is_contiguous()
+    n = ids.numel()
+    y = torch.empty(*ids.shape, weight.shape[1], dtype=BF16, device=weight.device)
+    check(lib.tlf_embedding(ids.data_ptr(), weight.data_ptr(), y.data_ptr(), n, weight.shape[0],
+                            weight.shape[1], _stream()), "tlf_embedding")
+    return y
+
+
+# ------------------------------------------------------------------ a10
+def w8a16_linear(x, wq, scale):
+    lib = _lib.load()
+    _need(x, BF16, "x"); _need(wq, torch.int8, "wq"); _need(scale, torch.float32, "scale")
+    assert x.stride(-1) == 1 and wq.is_contiguous()
+    x2 = x.reshape(-1, x.shape[-1])
+    M, K = x2.shape
+    N = wq.shape[0]
+    y = torch.empty(M, N, dtype=BF16, device=x.device)
+    nbytes = lib.tlf_w8a16_gemm_workspace_bytes(M, N, K)
+    ws = _workspace(nbytes, x.device, "gemm")
+    check(lib.tlf_w8a16_gemm(x2.data_ptr(), x2.stride(0), wq.data_ptr(), scale.data_ptr(), y.data_ptr(),
+                             M, N, K, ws.data_ptr(), ws.numel(), _stream()), "tlf_w8a16_gemm")
+    return y.view(*x.shape[:-1], N)
+
+
+def bf16_linear(x, w):
+    lib = _lib.load()
+    _need(x, BF16, "x"); _need(w, BF16, "w")
+    assert x.stride(-1) == 1 and w.is_contiguous()
+    x2 = x.reshape(-1, x.shape[-1])
+    M, K = x2.shape
+    N = w.shape[0]
+    y = torch.empty(M, N, dtype=BF16, device=x.device)
+    nbytes = lib.tlf_w8a16_gemm_workspace_bytes(M, N, K)
+    ws = _workspace(nbytes, x.device, "gemm")
+    check(lib.tlf_bf16_gemm(x2.data_ptr(), x2.stride(0), w.data_ptr(), y.data_ptr(), M, N, K,
+                            ws.data_ptr(), ws.numel(), _stream()), "tlf_bf16_gemm")
+    return y.view(*x.shape[:-1], N)
+
+
+# ------------------------------------------------------------------ a3
+def paged_decode_attention(q, k_cache, v_cache, context_lens, block_tables, scale,
+                           k_scale=None, v_scale=None):
+    """``q [B, Hq, Dh]`` -> ``[B, Hq*Dh]``; caches ``[nblk, bs, Hkv, Dh]``."""
+    lib = _lib.load()
+    _need(q, BF16, "q"); _need(context_lens, torch.int32, "context_lens")
+    _need(block_tables, torch.int32, "block_tables")
+    B, Hq, Dh = q.shape
+    assert q.stride(2) == 1 and q.stride(1) == Dh
+    nblk, bs, Hkv, _ = k_cache.shape
+    assert k_cache.is_contiguous() and v_cache.is_contiguous() and block_tables.stride(1) == 1
+    maxb = block_tables.shape[1]
+    out = torch.empty(B, Hq * Dh, dtype=BF16, device=q.device)
+    nbytes = lib.tlf_paged_decode_attn_workspace_bytes(B, Hq, Dh, maxb, bs)
+    ws = _workspace(nbytes, q.device, "decode")
+    check(lib.tlf_paged_decode_attn(
+        q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), kv_dtype_code(k_cache),
+        k_scale.data_ptr() if k_scale is not None else None,
+        v_scale.data_ptr() if v_scale is not None else None,
+        block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(), out.data_ptr(),
+        B, Hq, Hkv, Dh, bs, maxb, nblk, float(scale), ws.data_ptr(), ws.numel(), _stream()),
+        "tlf_paged_decode_attn")
+    return out
+
+
+# ------------------------------------------------------------------ a4
+def varlen_prefill_attention(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, scale,
+                             block_tables=None, k_scale=None, v_scale=None):
+    """``q [Sq, Hq, Dh]``; ``k``/``v`` packed ``[Sk, Hkv, Dh]`` or the paged caches with ``block_tables``."""
+    lib = _lib.load()
+    _need(q, BF16, "q"); _need(cu_seqlens_q, torch.int32, "cu_seqlens_q")
+    _need(cu_seqlens_k, torch.int32, "cu_seqlens_k")
+    Sq, Hq, Dh = q.shape
+    assert q.stride(2) == 1 and q.stride(1) == Dh
+    out = torch.empty(Sq, Hq * Dh, dtype=BF16, device=q.device)
+    nseq = cu_seqlens_q.numel() - 1
+    if block_tables is None:
+        _need(k, BF16, "k"); _need(v, BF16, "v")
+        Hkv = k.shape[1]
+        assert k.stride(2) == 1 and k.stride(1) == Dh and v.stride(2) == 1 and v.stride(1) == Dh
+        ks, vs, bs, nblk, kvd = k.stride(0), v.stride(0), 0, 0, KV_BF16
+        btp, bts = None, 0
+    else:
+        _need(block_tables, torch.int32, "block_tables")
+        nblk, bs, Hkv, _ = k.shape
+        assert k.is_contiguous() and v.is_contiguous()
+        ks = vs = Hkv * Dh
+        kvd = kv_dtype_code(k)
+        btp, bts = block_tables.data_ptr(), block_tables.stride(0)
+    check(lib.tlf_varlen_prefill_attn(
+        q.data_ptr(), q.stride(0), k.data_ptr(), ks, v.data_ptr(), vs, kvd,
+        k_scale.data_ptr() if k_scale is not None else None,
+        v_scale.data_ptr() if v_scale is not None else None,
+        cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr(), btp, bts, out.data_ptr(), nseq,
+        int(max_seqlen_q), Hq, Hkv, Dh, bs, nblk, float(scale), _stream()), "tlf_varlen_prefill_attn")
+    return out
