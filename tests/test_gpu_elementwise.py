@@ -158,14 +158,26 @@ def test_qknorm_rope_store_equals_unfused_sequence(ops, N, Hq, Hkv, want_kv):
     kc_ref, vc_ref = kc.clone(), vc.clone()
     O.store_kvcache(k_ref.view(N, Hkv, Dh), v.view(N, Hkv, Dh), kc_ref, vc_ref, slots)
     kc_d, vc_d = kc.to(DEV), vc.to(DEV)
-    qg, kg, vg = ops.qknorm_rope_store(qkv.to(DEV), qw.to(DEV), kw.to(DEV), 1e-6, pos.to(DEV), tab.to(DEV),
-                                       Hq, Hkv, Dh, kc_d, vc_d, slots.to(DEV), want_kv=want_kv)
-    assert_close_bf16(qg, q_ref, max_ulp=1.0, min_exact=0.99)
+    qkv_d, qw_d, kw_d, pos_d, tab_d, slots_d = (t.to(DEV) for t in (qkv, qw, kw, pos, tab, slots))
+    qg, kg, vg = ops.qknorm_rope_store(qkv_d, qw_d, kw_d, 1e-6, pos_d, tab_d, Hq, Hkv, Dh, kc_d, vc_d, slots_d,
+                                       want_kv=want_kv)
+    # (1) bit-identical to the unfused GPU kernels run one after the other
+    qd, kd, vd = qkv_d.split([Hq * Dh, Hkv * Dh, Hkv * Dh], dim=-1)
+    qn_d = ops.rms_norm(qd.view(N, Hq, Dh), qw_d, 1e-6).view(N, -1)
+    kn_d = ops.rms_norm(kd.view(N, Hkv, Dh), kw_d, 1e-6).view(N, -1)
+    qu, ku = ops.rope(pos_d, qn_d, kn_d, tab_d, Dh)
+    kc_u, vc_u = kc.to(DEV), vc.to(DEV)
+    ops.store_kvcache(ku.view(N, Hkv, Dh), vd.view(N, Hkv, Dh), kc_u, vc_u, slots_d)
+    assert torch.equal(qg, qu)
+    assert torch.equal(kc_d, kc_u) and torch.equal(vc_d, vc_u)
     if want_kv:
-        assert_close_bf16(kg, k_ref, max_ulp=1.0, min_exact=0.99)
+        assert torch.equal(kg, ku)
         assert torch.equal(vg.cpu().view(torch.int16), v.contiguous().view(torch.int16))
+    # (2) against the oracle: a 1-ulp difference after the norm (fp32 summation order) can grow to
+    # 2 ulp of a smaller rotated value, so allow 2 ulp here and require nearly all elements identical
+    assert_close_bf16(qg, q_ref, max_ulp=2.0, min_exact=0.99)
     assert torch.equal(vc_d.cpu().view(torch.int16), vc_ref.view(torch.int16))        # V rows are a bit copy
-    assert_close_bf16(kc_d, kc_ref, max_ulp=1.0, min_exact=0.99)
+    assert_close_bf16(kc_d, kc_ref, max_ulp=2.0, min_exact=0.99)
     # the cache holds exactly what the kernel returned for K, and untouched rows are untouched
     if want_kv:
         flat = kc_d.view(-1, Hkv * Dh)

@@ -1,0 +1,90 @@
+"""GPU parity: weight-only int8 linear and bf16 linear against the CPU oracle.
+
+Tolerance (north star): 2e-2 max-abs at bf16 output scale, 1e-3 relative L2.  With fp32
+accumulation only the summation order differs from the oracle, so the result must also be
+within one bf16 ulp everywhere.  Integer-valued activations make the W8A16 product exact
+in fp32, hence bit-exact.
+"""
+import pytest
+import torch
+
+from oracle import ops as O
+
+pytestmark = pytest.mark.gpu
+BF = torch.bfloat16
+DEV = "cuda"
+
+
+def g(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def make_w8(N, K, seed):
+    wq = torch.randint(-127, 128, (N, K), generator=g(seed), dtype=torch.int32).to(torch.int8)
+    scale = torch.rand(N, generator=g(seed + 1)) * 9e-3 + 1e-3
+    return wq, scale
+
+
+def check(got, ref_exact_fp32, ref_bf16, absdot):
+    """absdot = sum_k |x||w| (times the scale): fp32 accumulation in any order errs by at most
+    K * 2^-24 * absdot; 1e-6 * absdot covers that for K <= 16384 with room for the typical case."""
+    got = got.float().cpu()
+    rel = ((got - ref_bf16.float()).norm() / ref_bf16.float().norm()).item()
+    assert rel <= 1e-3, f"rel l2 {rel}"
+    err = (got - ref_exact_fp32).abs()
+    bound = O.bf16_ulp(ref_exact_fp32) + 1e-6 * absdot
+    assert (err <= bound).all(), f"max err/bound {(err / bound).max().item()}"
+    # max-abs 2e-2 is stated for O(1) outputs; scale it with the output magnitude
+    assert err.max().item() <= 2e-2 * max(1.0, ref_bf16.float().abs().max().item() / 4)
+
+
+SHAPES = [  # (M, N, K)
+    (1, 6144, 4096), (16, 4096, 4096), (64, 1024, 3072), (256, 4096, 4096), (300, 6144, 1024),
+    (512, 4096, 1024), (4, 1024, 2048), (2048, 1024, 1024), (257, 24576, 4096), (33, 4096, 12288),
+    (128, 5120, 8192), (7, 272, 64),
+]
+
+
+@pytest.mark.parametrize("M,N,K", SHAPES)
+def test_w8a16_gemm(M, N, K):
+    from tinyllmforge_amd import ops as P
+    x = torch.randn(M, K, generator=g(M + N)).to(BF)
+    wq, scale = make_w8(N, K, K)
+    exact = (x.double() @ wq.double().t()).float() * scale[None, :]
+    absdot = (x.double().abs() @ wq.double().abs().t()).float() * scale[None, :]
+    got = P.w8a16_linear(x.to(DEV), wq.to(DEV), scale.to(DEV))
+    assert got.shape == (M, N) and got.dtype == BF
+    check(got, exact, exact.to(BF), absdot)
+
+
+@pytest.mark.parametrize("M,N,K", [(5, 1024, 1024), (256, 4096, 4096), (130, 6144, 1024)])
+def test_w8a16_bit_exact_on_integer_activations(M, N, K):
+    from tinyllmforge_amd import ops as P
+    x = torch.randint(-4, 5, (M, K), generator=g(1)).to(BF)
+    wq, _ = make_w8(N, K, 2)
+    scale = torch.full((N,), 2.0 ** -9)
+    ref = O.w8a16_linear(x, wq, scale)
+    got = P.w8a16_linear(x.to(DEV), wq.to(DEV), scale.to(DEV)).cpu()
+    assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
+
+
+def test_w8a16_strided_activations_and_3d_input():
+    from tinyllmforge_amd import ops as P
+    M, N, K = 40, 1024, 1024
+    wide = torch.randn(M, K + 64, generator=g(3)).to(BF)
+    wq, scale = make_w8(N, K, 4)
+    got = P.w8a16_linear(wide.to(DEV)[:, :K], wq.to(DEV), scale.to(DEV))
+    exact = (wide[:, :K].double() @ wq.double().t()).float() * scale[None, :]
+    absdot = (wide[:, :K].double().abs() @ wq.double().abs().t()).float() * scale[None, :]
+    check(got, exact, exact.to(BF), absdot)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 1024), (4, 151936, 1024), (512, 4096, 1024), (256, 6144, 4096), (2048, 3072, 1024), (77, 1024, 3072)])
+def test_bf16_gemm(M, N, K):
+    from tinyllmforge_amd import ops as P
+    x = torch.randn(M, K, generator=g(M)).to(BF)
+    w = (torch.randn(N, K, generator=g(N)) * 0.05).to(BF)
+    exact = (x.double() @ w.double().t()).float()
+    absdot = (x.double().abs() @ w.double().abs().t()).float()
+    got = P.bf16_linear(x.to(DEV), w.to(DEV))
+    check(got, exact, exact.to(BF), absdot)

@@ -71,7 +71,8 @@ __global__ __launch_bounds__(NW * 64) void paged_decode_kernel(const DecodeParam
   __shared__ __attribute__((aligned(16))) unsigned short lds[NW][2][kTile][kLdsRow];
   const int b = blockIdx.y;
   const int part = blockIdx.x;
-  const int ctx = p.context_lens[b];
+  // a length beyond the table's capacity would overrun block_tables: clamp it
+  const int ctx = min(p.context_lens[b], p.max_blocks * p.block_size);
   const int t_begin = part * p.part_tokens;
   const int w = threadIdx.x >> 6;  // KV head
   const int lane = threadIdx.x & 63;
@@ -228,7 +229,7 @@ __global__ __launch_bounds__(64) void paged_decode_combine_kernel(const DecodePa
   const int b = blockIdx.y;
   const int head = blockIdx.x;
   const int lane = threadIdx.x;
-  const int ctx = p.context_lens[b];
+  const int ctx = min(p.context_lens[b], p.max_blocks * p.block_size);
   unsigned short *o = p.out + (static_cast<int64_t>(b) * p.num_q_heads + head) * kDh + lane * 2;
   if (ctx <= 0) {
     *reinterpret_cast<unsigned int *>(o) = 0u;
