@@ -102,6 +102,22 @@ def time_launches(fn, steps, warmup):
                 span_ms=span, wall_s=wall)
 
 
+def bench_probes(args):
+    """Rate of a plain read-only and a plain copy kernel over 1 GiB: the practical HBM ceiling of the box."""
+    import torch
+    from tinyllmforge_amd import _lib
+    lib = _lib.load()
+    n = 1 << 30
+    src = torch.empty(n, dtype=torch.uint8, device="cuda").random_(0, 255)
+    dst = torch.empty(n, dtype=torch.uint8, device="cuda")
+    sink = torch.zeros(1, dtype=torch.int32, device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    tr = time_launches(lambda: _lib.check(lib.tlf_probe_read(src.data_ptr(), n, sink.data_ptr(), st), "probe"), 30, 5)
+    tc = time_launches(lambda: _lib.check(lib.tlf_probe_copy(src.data_ptr(), dst.data_ptr(), n, st), "probe"), 30, 5)
+    return dict(read_GBps=round(n / (tr["mean_ms"] * 1e-3) / 1e9, 1),
+                copy_GBps=round(2 * n / (tc["mean_ms"] * 1e-3) / 1e9, 1), bytes=n)
+
+
 def bench_decode_attn(args):
     import torch
     from tinyllmforge_amd import ops as P
@@ -119,7 +135,7 @@ def bench_decode_attn(args):
     res = dict(ms_per_step=ms_per_step, value=gbps,
                roofline=dict(bound="hbm", achieved=round(kern_gbps, 1), peak=HBM_PEAK_GBPS, unit="GB/s",
                              frac=round(kern_gbps / HBM_PEAK_GBPS, 4), traffic=None,
-                             kernel="paged_decode_kernel<8> + paged_decode_combine_kernel",
+                             kernel="paged_decode_kernel<8,false> + paged_decode_merge_kernel",
                              launch_ms_mean=round(t["mean_ms"], 5), launch_ms_median=round(t["median_ms"], 5),
                              launch_ms_min=round(t["min_ms"], 5), algorithmic_bytes=case["algo_bytes"]),
                case=case)
@@ -191,6 +207,7 @@ def main():
     out = {}
     extra = {}
     res = bench_decode_attn(args)
+    extra["hbm_probe"] = bench_probes(args)
     if args.workload in ("gemm", "all"):
         extra["w8a16_gemm"] = bench_gemm(args)
     cpu = None

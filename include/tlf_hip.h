@@ -209,7 +209,9 @@ int tlf_bf16_gemm(const void *x, int64_t x_stride, const void *w, void *y,
  * context_lens int32 [batch]; a sequence with context_len <= 0 gets zeros.
  * out: bf16 [batch, Hq*Dh] contiguous.  fp32 softmax and accumulation, bf16
  * probabilities in the P.V product (as flash-attn does).
- * Dh == 128, Hq % Hkv == 0, Hq/Hkv <= 16, Hkv <= 16, block_size % 16 == 0.
+ * Dh == 128, Hq % Hkv == 0, Hq/Hkv <= 16, Hkv in {1,2,4,8,16}, block_size % 16 == 0,
+ * batch <= 1024.
+ * Calls that share a workspace must not overlap in time.
  */
 size_t tlf_paged_decode_attn_workspace_bytes(int32_t batch, int32_t num_q_heads,
                                              int32_t head_dim, int32_t max_blocks,
@@ -258,6 +260,16 @@ int tlf_varlen_prefill_attn(const void *q, int64_t q_stride,
  */
 int tlf_embedding(const int64_t *ids, const void *weight, void *y,
                   int32_t n, int32_t vocab, int32_t cols, void *stream);
+
+/* ---------------------------------------------------------------------------
+ * Bandwidth probes (no reference counterpart): plain streaming kernels that
+ * bench.py uses to measure the HBM rate a read-only / copy kernel reaches on
+ * the box and to scale the profiler's traffic counters.  bytes % 16 == 0,
+ * 16-byte aligned pointers; sink is a 4-byte device word that is never
+ * actually written for ordinary data.
+ */
+int tlf_probe_read(const void *src, size_t bytes, void *sink, void *stream);
+int tlf_probe_copy(const void *src, void *dst, size_t bytes, void *stream);
 
 #ifdef __cplusplus
 }

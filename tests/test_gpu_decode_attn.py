@@ -112,3 +112,36 @@ def test_decode_config2_shape_sampled_rows():
     case = make_case(0, B, 32, 8, 256, ctxs, 300, maxb=16)
     got, ref = run_both(case)
     check(got, ref)
+
+
+def test_decode_many_short_sequences_share_workgroups():
+    """Shares of the flat tile list span several sequences: boundaries, merges and direct rows mix."""
+    ge = torch.Generator().manual_seed(5)
+    ctxs = torch.randint(1, 70, (200,), generator=ge).tolist()
+    got, ref = run_both(make_case(21, len(ctxs), 16, 8, 256, ctxs, 210))
+    check(got, ref)
+
+
+def test_decode_repeated_calls_leave_counters_clean():
+    from tinyllmforge_amd import ops as P
+    case = make_case(23, 6, 32, 8, 256, [4096, 3000, 20, 1000, 4000, 2], 64, maxb=16)
+    q, kc, vc, cl, bt = [t.to(DEV) for t in case]
+    outs = [P.paged_decode_attention(q, kc, vc, cl, bt, 0.0884) for _ in range(4)]
+    for o in outs[1:]:
+        assert torch.equal(o, outs[0])
+    check(outs[0].cpu(), O.paged_decode_attention(*case, 0.0884))
+
+
+def test_decode_fp8_cache():
+    from tinyllmforge_amd import ops as P
+    Hkv, Dh = 8, 128
+    ctxs = [1, 16, 300, 2049, 777]
+    q, kc, vc, cl, bt = make_case(29, len(ctxs), 32, Hkv, 256, ctxs, 24)
+    ks = torch.rand(Hkv, generator=torch.Generator().manual_seed(1)) * 0.02 + 0.01
+    vs = torch.rand(Hkv, generator=torch.Generator().manual_seed(2)) * 0.02 + 0.01
+    k8 = O.quantize_fp8(kc.view(-1, Hkv, Dh), ks).view(kc.shape)
+    v8 = O.quantize_fp8(vc.view(-1, Hkv, Dh), vs).view(vc.shape)
+    ref = O.paged_decode_attention(q, k8, v8, cl, bt, 0.0884, ks, vs)
+    got = P.paged_decode_attention(q.to(DEV), k8.to(DEV), v8.to(DEV), cl.to(DEV), bt.to(DEV), 0.0884,
+                                   ks.to(DEV), vs.to(DEV)).cpu()
+    check(got, ref)

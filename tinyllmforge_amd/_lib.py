@@ -43,6 +43,8 @@ SIGNATURES = {
     "tlf_varlen_prefill_attn": (c_int32, [_P, _I64, _P, _I64, _P, _I64, _I32, _P, _P, _P, _P, _P, _I64,
                                           _P, _I32, _I32, _I32, _I32, _I32, _I32, _I64, _F, _P]),
     "tlf_embedding": (c_int32, [_P, _P, _P, _I32, _I32, _I32, _P]),
+    "tlf_probe_read": (c_int32, [_P, _SZ, _P, _P]),
+    "tlf_probe_copy": (c_int32, [_P, _P, _SZ, _P]),
 }
 
 

@@ -62,6 +62,15 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
   return p;
 }
 
+// 128-bit load with the non-temporal hint: data that is read once (KV-cache rows,
+// weights at small batch) should not displace L2 / Infinity Cache lines; on MI355X a
+// read-only stream is ~10% faster with it (measured: 7.1 vs 6.3 TB/s).
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 load_nt_u4(const void *p) {
+  const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);

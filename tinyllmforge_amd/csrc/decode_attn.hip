@@ -3,30 +3,36 @@
 // token per sequence).
 //
 // HBM-bound streaming kernel.  A K (or V) cache row of one token holds all KV
-// heads contiguously (Hkv * 128 bf16 = 2 KiB), so one workgroup owns a run of
-// tokens of one sequence and ALL its KV heads: wave w <-> KV head w.  Together
-// the waves read whole contiguous rows with 128-bit loads, and the Hq/Hkv query
-// heads that share a KV head are served from a single pass over its rows
-// (GQA sharing), so every cache byte is fetched exactly once.
+// heads contiguously (Hkv * 128 bf16 = 2 KiB), so a workgroup owns a run of
+// tokens and ALL KV heads: wave w <-> KV head w.  Together the waves read whole
+// contiguous rows with 128-bit loads, and the Hq/Hkv query heads that share a KV
+// head are served from one pass over its rows (GQA sharing): every cache byte is
+// fetched exactly once.
+//
+// Work split (data-independent grid, so the launch can be graph-captured):
+// the 16-token tiles of all sequences form one flat list; the G persistent
+// workgroups take equal contiguous shares of it (computed on the device from
+// context_lens by a block scan), so every workgroup streams the same number of
+// bytes whatever the mix of lengths.  A share may cover the end of one sequence
+// and the start of the next.  A sequence that lies inside one share is finished
+// there; a sequence cut by share boundaries gets one partial (max, sum,
+// unnormalised O) per share, and a small second kernel merges the partials of
+// the cut sequences.  (Merging inside the first kernel needs device-scope
+// fences, i.e. an L2 write-back and invalidate per workgroup on this multi-XCD
+// part: measured at +80 us on a 120 us kernel, against ~5 us for the second
+// launch.)
 //
 // Per wave and 16-token tile:
-//   global (4 x 128-bit loads per lane for K, 4 for V, issued one tile ahead)
-//     -> LDS (row-major [token][dim], padded rows)
+//   global (128-bit loads, issued one tile ahead) -> LDS (row-major, padded rows)
 //   S^T[token, head] = K_tile . Q^T        4 x v_mfma_f32_16x16x32_bf16
 //   online softmax in fp32 (row max / sum by two cross-lane exchanges)
-//   O^T[dim, head]  += V_tile^T . P^T      8 x v_mfma_f32_16x16x16_bf16
+//   O^T[dim, head]  += V_tile^T . P^T      v_mfma_f32_16x16x16_bf16; the V^T operand is
+//                                          read from the row-major tile by ds_read_b64_tr_b16
 // The MFMA output layout of S^T (lane = head, 4 tokens per lane) is exactly the
 // B-operand layout of the second product, so P never leaves registers, and the
 // softmax statistics of a head live in the lanes that hold its O^T columns.
 // P is fed as a bf16 hi + lo pair (two MFMAs): matrix-core time is free in a
 // bandwidth-bound kernel and it removes the bf16 rounding of the probabilities.
-//
-// Long sequences are cut into fixed-size partitions (grid = partitions x
-// batch, independent of device data, so the launch can be graph-captured);
-// partitions beyond a sequence's length exit at once.  Each partition writes
-// (max, sum, unnormalised O) and a small second kernel merges them.
-#include <stdlib.h>
-
 #include "common.h"
 
 namespace tlf {
@@ -34,6 +40,9 @@ namespace tlf {
 constexpr int kDh = 128;
 constexpr int kTile = 16;             // tokens per tile
 constexpr int kLdsRow = kDh + 8;      // padded LDS row (elements): 272 B, shifts rows by 4 banks
+constexpr int kMaxBatch = 1024;       // sequences per call (prefix table lives in LDS)
+constexpr int kMinTiles = 4;          // smallest share of a workgroup, in tiles
+constexpr int kMaxGrid = 1024;        // workspace is sized for this many workgroups
 constexpr float kLog2e = 1.4426950408889634f;
 
 struct DecodeParams {
@@ -47,231 +56,359 @@ struct DecodeParams {
   int64_t bt_stride;
   const int32_t *context_lens;
   unsigned short *out;
-  float *part_o;   // [batch, nparts, Hq, 128]
-  float *part_ml;  // [batch, nparts, Hq, 2]  (max in log2 domain, sum)
+  int32_t *meta;      // [batch, 2]: first workgroup and number of shares of each sequence
+  float *part_ml;     // [slots, Hq, 2]  (max in log2 domain, sum)
+  float *part_o;      // [slots, Hq, 128]
+  int32_t batch;
   int32_t num_q_heads;
   int32_t num_kv_heads;
   int32_t block_size;
   int32_t max_blocks;
   int64_t num_cache_blocks;
-  int32_t part_tokens;
-  int32_t nparts;
   float scale_log2;  // softmax scale * log2(e)
 };
 
-// One tile's worth of global data of one wave: 16 tokens x 128 dims of K and V.
+__device__ __forceinline__ shortx4 lds_read_tr16_b64(const unsigned short *p) {
+  // within each group of 16 lanes, lane i receives {row0[i], row1[i], row2[i], row3[i]},
+  // row j being the 16 elements addressed (4 each) by lanes 4j .. 4j+3 of the group
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (shortx4 __attribute__((address_space(3))) *)(p));
+}
+
+__device__ __forceinline__ void fp8x16_to_bf16x16(const uint4 &in, uint4 &lo, uint4 &hi) {
+  auto cv = [](unsigned int w, unsigned int &a, unsigned int &b) {
+    const auto f0 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w), false);
+    const auto f1 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w), true);
+    a = pack_bf16x2(f0[0], f0[1]);
+    b = pack_bf16x2(f1[0], f1[1]);
+  };
+  cv(in.x, lo.x, lo.y);
+  cv(in.y, lo.z, lo.w);
+  cv(in.z, hi.x, hi.y);
+  cv(in.w, hi.z, hi.w);
+}
+
+// One tile's worth of global data of one wave: 16 tokens x 128 dims of K and V
+// (4 + 4 128-bit loads per lane for bf16, 2 + 2 for e4m3).
+template <bool KV8>
 struct TileRegs {
-  uint4 k[4];
-  uint4 v[4];
+  static constexpr int kLoads = KV8 ? 2 : 4;
+  uint4 k[kLoads];
+  uint4 v[kLoads];
   bool ok;  // the tile's block-table entry names a real cache block
 };
 
-template <int NW>
-__global__ __launch_bounds__(NW * 64) void paged_decode_kernel(const DecodeParams p) {
+template <int NW, bool KV8>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void paged_decode_kernel(const DecodeParams p) {
+  constexpr int kThreads = NW * 64;
   __shared__ __attribute__((aligned(16))) unsigned short lds[NW][2][kTile][kLdsRow];
-  const int b = blockIdx.y;
-  const int part = blockIdx.x;
-  // a length beyond the table's capacity would overrun block_tables: clamp it
-  const int ctx = min(p.context_lens[b], p.max_blocks * p.block_size);
-  const int t_begin = part * p.part_tokens;
-  const int w = threadIdx.x >> 6;  // KV head
-  const int lane = threadIdx.x & 63;
+  __shared__ int s_prefix[kMaxBatch + 1];  // tiles before sequence b
+  __shared__ int s_wave_tot[16];
+  __shared__ int s_start_b;
+
+  const int tid = threadIdx.x;
+  const int w = tid >> 6;  // KV head
+  const int lane = tid & 63;
   const int n = lane & 15;  // query head inside the group (MFMA column)
   const int g = lane >> 4;
   const int group = p.num_q_heads / p.num_kv_heads;
   const int head = w * group + n;
   const bool head_ok = n < group;
+  const int max_ctx = p.max_blocks * p.block_size;  // a longer length would overrun the table
 
-  if (t_begin >= ctx) {
-    if (p.nparts == 1 && head_ok) {  // empty sequence: zeros, nobody else writes this row
-      unsigned short *o = p.out + (static_cast<int64_t>(b) * p.num_q_heads + head) * kDh;
-#pragma unroll
-      for (int d = 0; d < 8; ++d)
-        *reinterpret_cast<uint2 *>(o + d * 16 + g * 4) = make_uint2(0, 0);
+  // ---- 1. tiles per sequence -> exclusive prefix in LDS (block scan, chunks of kThreads)
+  if (tid == 0) s_prefix[0] = 0;
+  int carry = 0;
+  for (int base = 0; base < p.batch; base += kThreads) {
+    const int b = base + tid;
+    int tiles = 0;
+    if (b < p.batch) {
+      const int c = min(p.context_lens[b], max_ctx);
+      tiles = c > 0 ? (c + kTile - 1) / kTile : 0;
     }
-    return;
-  }
-  const int t_end = min(ctx, t_begin + p.part_tokens);
-
-  // Q as the B operand of S^T = K . Q^T: lane (n, g) holds q[head n][c*32 + g*8 .. +8].
-  bf16x8 qf[4];
-  {
-    const unsigned short *qp = p.q + b * p.q_stride + static_cast<int64_t>(head) * kDh;
+    int incl = tiles;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      Pack16 t;
-      t.u = make_uint4(0, 0, 0, 0);
-      if (head_ok) t.u = *reinterpret_cast<const uint4 *>(qp + c * 32 + g * 8);
-      qf[c] = t.v;
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += up;
     }
+    if (lane == 63) s_wave_tot[w] = incl;
+    __syncthreads();
+    int before = carry;
+    for (int ww = 0; ww < w; ++ww) before += s_wave_tot[ww];
+    if (b < p.batch) s_prefix[b + 1] = before + incl;
+    int total = 0;
+    for (int ww = 0; ww < NW; ++ww) total += s_wave_tot[ww];
+    carry += total;
+    __syncthreads();
   }
+  const int total_tiles = carry;
 
-  const int64_t row_elems = static_cast<int64_t>(p.num_kv_heads) * kDh;
-  const int32_t *bt = p.block_tables + b * p.bt_stride;
-  unsigned short(*Ks)[kLdsRow] = lds[w][0];
-  unsigned short(*Vs)[kLdsRow] = lds[w][1];
-
-  // Issue the loads of the tile starting at token t0 (a tile never straddles a block).
-  auto load_tile = [&](int t0, TileRegs &r) {
-    const int bi = t0 / p.block_size;
-    const int64_t blk = bt[bi];
-    const bool ok = blk >= 0 && blk < p.num_cache_blocks;
-    const int64_t tok0 = (ok ? blk : 0) * p.block_size + (t0 - bi * p.block_size);
-    r.ok = ok;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int tt = i * 4 + g;  // token of this lane inside the tile
-      const int64_t off = ((tok0 + tt) * row_elems + w * kDh + n * 8) * 2;
-      const bool valid = ok && (t0 + tt) < t_end;
-      r.k[i] = make_uint4(0, 0, 0, 0);
-      r.v[i] = make_uint4(0, 0, 0, 0);
-      if (valid) {
-        r.k[i] = *reinterpret_cast<const uint4 *>(p.k_cache + off);
-        r.v[i] = *reinterpret_cast<const uint4 *>(p.v_cache + off);
+  // ---- 2. empty sequences get zeros (workgroup 0 owns that)
+  if (blockIdx.x == 0) {
+    for (int b = 0; b < p.batch; ++b) {
+      if (s_prefix[b + 1] == s_prefix[b]) {
+        if (tid == 0) *reinterpret_cast<int2 *>(p.meta + 2 * b) = make_int2(0, 0);
+        unsigned short *o = p.out + static_cast<int64_t>(b) * p.num_q_heads * kDh;
+        for (int i = tid * 8; i < p.num_q_heads * kDh; i += kThreads * 8)
+          *reinterpret_cast<uint4 *>(o + i) = make_uint4(0, 0, 0, 0);
       }
     }
-  };
-
-  floatx4 acc[8];
-#pragma unroll
-  for (int d = 0; d < 8; ++d) acc[d] = floatx4{0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY;  // running max (log2 domain), identical in the 4 lanes of a head
-  float l_run = 0.f;        // this lane's share of the running sum
-
-  TileRegs regs;
-  load_tile(t_begin, regs);
-  for (int t0 = t_begin; t0 < t_end; t0 += kTile) {
-    wave_lds_fence();  // previous tile's LDS reads are done
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      *reinterpret_cast<uint4 *>(&Ks[i * 4 + g][n * 8]) = regs.k[i];
-      *reinterpret_cast<uint4 *>(&Vs[i * 4 + g][n * 8]) = regs.v[i];
-    }
-    wave_lds_fence();
-    const bool tile_ok = regs.ok;
-    if (t0 + kTile < t_end) load_tile(t0 + kTile, regs);
-
-    // S^T = K . Q^T : lane (n, g) gets tokens g*4 + i of head n
-    floatx4 s = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-      Pack16 a;
-      a.u = *reinterpret_cast<const uint4 *>(&Ks[n][c * 32 + g * 8]);
-      s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[c], s, 0, 0, 0);
-    }
-    float sv[4];
-    float mt = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const bool valid = tile_ok && (t0 + g * 4 + i) < t_end;
-      sv[i] = valid ? s[i] * p.scale_log2 : -INFINITY;
-      mt = fmaxf(mt, sv[i]);
-    }
-    mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-    mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-    const float m_new = fmaxf(m_run, mt);
-    // -inf only while every token so far sat in a skipped block: keep the exponents finite
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = exp2f(m_run - m_use);
-    float psum = 0.f;
-    bf16x4 pb, pl;  // p = hi + lo in bf16: the matrix cores are idle here, so P.V keeps ~16 bits of p
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float pv = exp2f(sv[i] - m_use);
-      psum += pv;
-      pb[i] = static_cast<__bf16>(pv);
-      pl[i] = static_cast<__bf16>(pv - static_cast<float>(pb[i]));
-    }
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
-    const shortx4 pbs = __builtin_bit_cast(shortx4, pb);
-    const shortx4 pls = __builtin_bit_cast(shortx4, pl);
-#pragma unroll
-    for (int d = 0; d < 8; ++d) {
-      // A = V^T fragment: lane (dim = d*16 + n, g) holds tokens g*4 + i
-      shortx4 vf;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) vf[i] = static_cast<short>(Vs[g * 4 + i][d * 16 + n]);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) acc[d][i] *= alpha;
-      acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pbs, acc[d], 0, 0, 0);
-      acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pls, acc[d], 0, 0, 0);
-    }
   }
 
-  l_run += __shfl_xor(l_run, 16, 64);
-  l_run += __shfl_xor(l_run, 32, 64);
-  if (!head_ok) return;
-  // lane (n, g) holds O^T[dims d*16 + g*4 + i][head n]
-  if (p.nparts == 1) {
-    const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
-    unsigned short *o = p.out + (static_cast<int64_t>(b) * p.num_q_heads + head) * kDh;
+  // ---- 3. this workgroup's share [ts, te) of the flat tile list
+  const int G = gridDim.x;
+  int tpw = (total_tiles + G - 1) / G;
+  if (tpw < kMinTiles) tpw = kMinTiles;
+  const int ts = blockIdx.x * tpw;
+  const int te = min(total_tiles, ts + tpw);
+  if (ts >= total_tiles) return;  // uniform
+  for (int b = tid; b < p.batch; b += kThreads)
+    if (s_prefix[b] <= ts && ts < s_prefix[b + 1]) s_start_b = b;
+  __syncthreads();
+
+  const int64_t row_elems = static_cast<int64_t>(p.num_kv_heads) * kDh;
+  unsigned short(*Ks)[kLdsRow] = lds[w][0];
+  unsigned short(*Vs)[kLdsRow] = lds[w][1];
+  const float kscale = KV8 ? p.k_scale[w] : 1.0f;
+  const float vscale = KV8 ? p.v_scale[w] : 1.0f;
+  const float scale_log2 = p.scale_log2 * kscale;
+
+  int b = s_start_b;
+  int cur = ts;
+  while (cur < te) {
+    while (s_prefix[b + 1] <= cur) ++b;  // skip empty sequences (uniform)
+    const int seq_first = s_prefix[b];
+    const int seq_end = s_prefix[b + 1];
+    const int seg_end = min(te, seq_end);
+    const int ctx = min(p.context_lens[b], max_ctx);
+    const int t_begin = (cur - seq_first) * kTile;
+    const int t_end = min(ctx, (seg_end - seq_first) * kTile);
+
+    // Q as the B operand of S^T = K . Q^T: lane (n, g) holds q[head n][c*32 + g*8 .. +8].
+    bf16x8 qf[4];
+    {
+      const unsigned short *qp = p.q + b * p.q_stride + static_cast<int64_t>(head) * kDh;
 #pragma unroll
-    for (int d = 0; d < 8; ++d) {
-      uint2 st;
-      st.x = pack_bf16x2(acc[d][0] * inv, acc[d][1] * inv);
-      st.y = pack_bf16x2(acc[d][2] * inv, acc[d][3] * inv);
-      *reinterpret_cast<uint2 *>(o + d * 16 + g * 4) = st;
+      for (int c = 0; c < 4; ++c) {
+        Pack16 t;
+        t.u = make_uint4(0, 0, 0, 0);
+        if (head_ok) t.u = *reinterpret_cast<const uint4 *>(qp + c * 32 + g * 8);
+        qf[c] = t.v;
+      }
     }
-  } else {
-    const int64_t slot = (static_cast<int64_t>(b) * p.nparts + part) * p.num_q_heads + head;
-    float *po = p.part_o + slot * kDh;
+    const int32_t *bt = p.block_tables + b * p.bt_stride;
+
+    // Issue the loads of the tile starting at token t0 (a tile never straddles a block);
+    // blk is its block-table entry, fetched one tile earlier so that its latency is hidden.
+    auto load_tile = [&](int t0, int64_t blk, TileRegs<KV8> &r) {
+      const int bi = t0 / p.block_size;
+      const bool ok = blk >= 0 && blk < p.num_cache_blocks;
+      const int64_t tok0 = (ok ? blk : 0) * p.block_size + (t0 - bi * p.block_size);
+      r.ok = ok;
 #pragma unroll
-    for (int d = 0; d < 8; ++d)
-      *reinterpret_cast<float4 *>(po + d * 16 + g * 4) =
-          make_float4(acc[d][0], acc[d][1], acc[d][2], acc[d][3]);
-    if (g == 0) *reinterpret_cast<float2 *>(p.part_ml + slot * 2) = make_float2(m_run, l_run);
+      for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
+        // bf16: 4 tokens x 16 chunks of 8 elements per instruction; e4m3: 8 tokens x 8 chunks of 16
+        const int tt = KV8 ? i * 8 + (lane >> 3) : i * 4 + g;
+        const int64_t off = KV8 ? (tok0 + tt) * row_elems + w * kDh + (lane & 7) * 16
+                                : ((tok0 + tt) * row_elems + w * kDh + n * 8) * 2;
+        const bool valid = ok && (t0 + tt) < t_end;
+        r.k[i] = make_uint4(0, 0, 0, 0);
+        r.v[i] = make_uint4(0, 0, 0, 0);
+        if (valid) {
+          r.k[i] = load_nt_u4(p.k_cache + off);
+          r.v[i] = load_nt_u4(p.v_cache + off);
+        }
+      }
+    };
+    auto store_tile = [&](const TileRegs<KV8> &r) {
+#pragma unroll
+      for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
+        if (KV8) {
+          const int tt = i * 8 + (lane >> 3);
+          const int ch = (lane & 7) * 16;
+          uint4 lo, hi;
+          fp8x16_to_bf16x16(r.k[i], lo, hi);
+          *reinterpret_cast<uint4 *>(&Ks[tt][ch]) = lo;
+          *reinterpret_cast<uint4 *>(&Ks[tt][ch + 8]) = hi;
+          fp8x16_to_bf16x16(r.v[i], lo, hi);
+          *reinterpret_cast<uint4 *>(&Vs[tt][ch]) = lo;
+          *reinterpret_cast<uint4 *>(&Vs[tt][ch + 8]) = hi;
+        } else {
+          *reinterpret_cast<uint4 *>(&Ks[i * 4 + g][n * 8]) = r.k[i];
+          *reinterpret_cast<uint4 *>(&Vs[i * 4 + g][n * 8]) = r.v[i];
+        }
+      }
+    };
+
+    floatx4 acc[8];
+#pragma unroll
+    for (int d = 0; d < 8; ++d) acc[d] = floatx4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY;  // running max (log2 domain), identical in the 4 lanes of a head
+    float l_run = 0.f;        // this lane's share of the running sum
+
+    TileRegs<KV8> regs;
+    load_tile(t_begin, bt[t_begin / p.block_size], regs);
+    // block-table entry of the tile after this one (clamped to the segment: never read beyond it)
+    int next_blk = bt[min(t_begin + kTile, t_end - 1) / p.block_size];
+    for (int t0 = t_begin; t0 < t_end; t0 += kTile) {
+      wave_lds_fence();  // previous tile's LDS reads are done
+      store_tile(regs);
+      wave_lds_fence();
+      const bool tile_ok = regs.ok;
+      if (t0 + kTile < t_end) {
+        load_tile(t0 + kTile, next_blk, regs);
+        next_blk = bt[min(t0 + 2 * kTile, t_end - 1) / p.block_size];
+      }
+
+      // S^T = K . Q^T : lane (n, g) gets tokens g*4 + i of head n
+      floatx4 s = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        Pack16 a;
+        a.u = *reinterpret_cast<const uint4 *>(&Ks[n][c * 32 + g * 8]);
+        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[c], s, 0, 0, 0);
+      }
+      float sv[4];
+      float mt = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const bool valid = tile_ok && (t0 + g * 4 + i) < t_end;
+        sv[i] = valid ? s[i] * scale_log2 : -INFINITY;
+        mt = fmaxf(mt, sv[i]);
+      }
+      mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+      const float m_new = fmaxf(m_run, mt);
+      // -inf only while every token so far sat in a skipped block: keep the exponents finite
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = exp2f(m_run - m_use);
+      float psum = 0.f;
+      bf16x4 pb, pl;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pv = exp2f(sv[i] - m_use);
+        psum += pv;
+        pb[i] = static_cast<__bf16>(pv);
+        pl[i] = static_cast<__bf16>(pv - static_cast<float>(pb[i]));
+      }
+      l_run = l_run * alpha + psum;
+      m_run = m_new;
+      const shortx4 pbs = __builtin_bit_cast(shortx4, pb);
+      const shortx4 pls = __builtin_bit_cast(shortx4, pl);
+#pragma unroll
+      for (int d = 0; d < 8; ++d) {
+        // A = V^T fragment: lane (dim = d*16 + n, g) <- tokens g*4 + 0..3 (transpose read)
+        const shortx4 vf = lds_read_tr16_b64(&Vs[g * 4 + (n >> 2)][d * 16 + (n & 3) * 4]);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[d][i] *= alpha;
+        acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pbs, acc[d], 0, 0, 0);
+        acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pls, acc[d], 0, 0, 0);
+      }
+    }
+    l_run += __shfl_xor(l_run, 16, 64);
+    l_run += __shfl_xor(l_run, 32, 64);
+
+    // ---- finish the segment.  lane (n, g) holds O^T[dims d*16 + g*4 + i][head n]
+    const int w_first = seq_first / tpw;
+    const int w_last = (seq_end - 1) / tpw;
+    const int nseg = w_last - w_first + 1;
+    if (nseg == 1) {
+      if (head_ok) {
+        const float inv = l_run > 0.f ? vscale / l_run : 0.f;
+        unsigned short *o = p.out + (static_cast<int64_t>(b) * p.num_q_heads + head) * kDh;
+#pragma unroll
+        for (int d = 0; d < 8; ++d) {
+          uint2 st;
+          st.x = pack_bf16x2(acc[d][0] * inv, acc[d][1] * inv);
+          st.y = pack_bf16x2(acc[d][2] * inv, acc[d][3] * inv);
+          *reinterpret_cast<uint2 *>(o + d * 16 + g * 4) = st;
+        }
+      }
+    } else {
+      // (workgroup, sequence) pairs form a staircase, so blockIdx + b is a unique slot
+      const int64_t slot = (static_cast<int64_t>(blockIdx.x) + b) * p.num_q_heads;
+      if (head_ok) {
+        float *po = p.part_o + (slot + head) * kDh;
+#pragma unroll
+        for (int d = 0; d < 8; ++d)
+          *reinterpret_cast<float4 *>(po + d * 16 + g * 4) =
+              make_float4(acc[d][0] * vscale, acc[d][1] * vscale, acc[d][2] * vscale,
+                          acc[d][3] * vscale);
+        if (g == 0) *reinterpret_cast<float2 *>(p.part_ml + (slot + head) * 2) = make_float2(m_run, l_run);
+      }
+    }
+    if (tid == 0 && cur == seq_first)  // the share holding the sequence's first tile records its split
+      *reinterpret_cast<int2 *>(p.meta + 2 * b) = make_int2(w_first, nseg);
+    cur = seg_end;
+    ++b;
   }
 }
 
-// Merge the partitions of one (sequence, head): one wave, two dims per lane.
-__global__ __launch_bounds__(64) void paged_decode_combine_kernel(const DecodeParams p) {
+// Merge the partials of the sequences that were cut by share boundaries.
+// grid = (Hq / 8, batch); a thread owns 4 dims of one head and walks the shares
+// four at a time, so that 8 independent loads are in flight per step (the loop is
+// latency bound: partials were just written by other CUs).
+__global__ __launch_bounds__(256) void paged_decode_merge_kernel(const DecodeParams p) {
   const int b = blockIdx.y;
-  const int head = blockIdx.x;
-  const int lane = threadIdx.x;
-  const int ctx = min(p.context_lens[b], p.max_blocks * p.block_size);
-  unsigned short *o = p.out + (static_cast<int64_t>(b) * p.num_q_heads + head) * kDh + lane * 2;
-  if (ctx <= 0) {
-    *reinterpret_cast<unsigned int *>(o) = 0u;
-    return;
-  }
-  const int np = min(p.nparts, (ctx + p.part_tokens - 1) / p.part_tokens);
-  const int64_t base = (static_cast<int64_t>(b) * p.nparts) * p.num_q_heads + head;
-  float m = -INFINITY;
-  for (int i = 0; i < np; ++i)
-    m = fmaxf(m, p.part_ml[(base + static_cast<int64_t>(i) * p.num_q_heads) * 2]);
-  float l = 0.f, a0 = 0.f, a1 = 0.f;
-  for (int i = 0; i < np; ++i) {
-    const int64_t slot = base + static_cast<int64_t>(i) * p.num_q_heads;
-    const float2 ml = *reinterpret_cast<const float2 *>(p.part_ml + slot * 2);
-    const float wgt = (ml.x == -INFINITY) ? 0.f : exp2f(ml.x - m);
-    const float2 v = *reinterpret_cast<const float2 *>(p.part_o + slot * kDh + lane * 2);
-    l += wgt * ml.y;
-    a0 += wgt * v.x;
-    a1 += wgt * v.y;
-  }
-  const float inv = l > 0.f ? 1.0f / l : 0.f;
-  *reinterpret_cast<unsigned int *>(o) = pack_bf16x2(a0 * inv, a1 * inv);
-}
-
-inline int decode_part_tokens() {
-  static int cached = 0;
-  if (cached == 0) {
-    int v = 256;
-    if (const char *e = getenv("TLF_DECODE_PART_TOKENS")) {
-      const int x = atoi(e);
-      if (x >= kTile && x % kTile == 0) v = x;
+  const int2 meta = *reinterpret_cast<const int2 *>(p.meta + 2 * b);
+  const int w_first = meta.x, nseg = meta.y;
+  if (nseg <= 1) return;  // finished by the first kernel (or empty)
+  const int hh = blockIdx.x * 8 + (threadIdx.x >> 5);
+  if (hh >= p.num_q_heads) return;
+  const int c4 = (threadIdx.x & 31) * 4;
+  const int64_t base = (static_cast<int64_t>(w_first) + b) * p.num_q_heads + hh;
+  float M = -INFINITY, L = 0.f;
+  float4 A = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int s0 = 0; s0 < nseg; s0 += 4) {
+    float2 ml[4];
+    float4 o4[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int s = min(s0 + u, nseg - 1);  // clamped duplicate gets weight 0 below
+      const int64_t sl = base + static_cast<int64_t>(s) * p.num_q_heads;
+      ml[u] = *reinterpret_cast<const float2 *>(p.part_ml + sl * 2);
+      o4[u] = *reinterpret_cast<const float4 *>(p.part_o + sl * kDh + c4);
     }
-    cached = v;
+    float Mn = M;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (s0 + u < nseg) Mn = fmaxf(Mn, ml[u].x);
+    if (Mn == -INFINITY) continue;
+    const float a = exp2f(M - Mn);
+    L *= a;
+    A.x *= a; A.y *= a; A.z *= a; A.w *= a;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const float wgt = (s0 + u < nseg && ml[u].x != -INFINITY) ? exp2f(ml[u].x - Mn) : 0.f;
+      L += wgt * ml[u].y;
+      A.x += wgt * o4[u].x;
+      A.y += wgt * o4[u].y;
+      A.z += wgt * o4[u].z;
+      A.w += wgt * o4[u].w;
+    }
+    M = Mn;
   }
-  return cached;
+  const float inv = L > 0.f ? 1.0f / L : 0.f;
+  uint2 st;
+  st.x = pack_bf16x2(A.x * inv, A.y * inv);
+  st.y = pack_bf16x2(A.z * inv, A.w * inv);
+  *reinterpret_cast<uint2 *>(p.out + (static_cast<int64_t>(b) * p.num_q_heads + hh) * kDh + c4) = st;
 }
 
-inline int decode_nparts(int32_t max_blocks, int32_t block_size) {
-  const int64_t max_tokens = static_cast<int64_t>(max_blocks) * block_size;
-  const int pt = decode_part_tokens();
-  return static_cast<int>((max_tokens + pt - 1) / pt);
+inline int device_cu_count() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess)
+      cus = prop.multiProcessorCount;
+    if (cus <= 0) cus = 256;
+  }
+  return cus;
 }
+
+inline size_t decode_meta_bytes() { return 2 * kMaxBatch * sizeof(int32_t); }
 
 }  // namespace tlf
 
@@ -280,11 +417,12 @@ using namespace tlf;
 extern "C" size_t tlf_paged_decode_attn_workspace_bytes(int32_t batch, int32_t num_q_heads,
                                                         int32_t head_dim, int32_t max_blocks,
                                                         int32_t block_size) {
-  if (batch <= 0 || num_q_heads <= 0 || head_dim <= 0 || max_blocks <= 0 || block_size <= 0)
-    return 0;
-  const size_t np = static_cast<size_t>(decode_nparts(max_blocks, block_size));
-  const size_t slots = static_cast<size_t>(batch) * np * num_q_heads;
-  return slots * (static_cast<size_t>(head_dim) + 2) * sizeof(float) + 256;
+  (void)max_blocks;
+  (void)block_size;
+  if (batch <= 0 || num_q_heads <= 0 || head_dim <= 0) return 0;
+  const size_t slots = static_cast<size_t>(kMaxGrid) + batch;
+  return decode_meta_bytes() +
+         slots * num_q_heads * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
 }
 
 extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void *k_cache,
@@ -298,19 +436,23 @@ extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void
   if (batch == 0) return TLF_OK;
   if (!q || !k_cache || !v_cache || !block_tables || !context_lens || !out) return TLF_E_NULL;
   if (head_dim != kDh) return TLF_E_UNSUPPORTED;
-  if (kv_dtype != TLF_KV_BF16) return TLF_E_UNSUPPORTED;
-  if (batch < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || block_size <= 0 || max_blocks <= 0 ||
-      num_cache_blocks <= 0)
+  if (kv_dtype != TLF_KV_BF16 && kv_dtype != TLF_KV_FP8_E4M3) return TLF_E_UNSUPPORTED;
+  if (kv_dtype == TLF_KV_FP8_E4M3 && (!k_scale || !v_scale)) return TLF_E_NULL;
+  if (batch < 0 || batch > kMaxBatch || num_q_heads <= 0 || num_kv_heads <= 0 || block_size <= 0 ||
+      max_blocks <= 0 || num_cache_blocks <= 0)
     return TLF_E_SHAPE;
   if (num_q_heads % num_kv_heads || num_q_heads / num_kv_heads > 16 || block_size % kTile)
     return TLF_E_SHAPE;
+  if (static_cast<int64_t>(max_blocks) * block_size > (1ll << 30)) return TLF_E_SHAPE;
   if (block_table_stride < max_blocks || q_stride < static_cast<int64_t>(num_q_heads) * head_dim)
     return TLF_E_SHAPE;
   if (!aligned16(q) || q_stride % 8 || !aligned16(k_cache) || !aligned16(v_cache) ||
       !aligned16(out))
     return TLF_E_ALIGN;
-  (void)k_scale;
-  (void)v_scale;
+  const size_t need =
+      tlf_paged_decode_attn_workspace_bytes(batch, num_q_heads, head_dim, max_blocks, block_size);
+  if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+    return TLF_E_WORKSPACE;
 
   DecodeParams p;
   p.q = static_cast<const unsigned short *>(q);
@@ -323,40 +465,45 @@ extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void
   p.bt_stride = block_table_stride;
   p.context_lens = context_lens;
   p.out = static_cast<unsigned short *>(out);
+  p.batch = batch;
   p.num_q_heads = num_q_heads;
   p.num_kv_heads = num_kv_heads;
   p.block_size = block_size;
   p.max_blocks = max_blocks;
   p.num_cache_blocks = num_cache_blocks;
-  p.part_tokens = decode_part_tokens();
-  p.nparts = decode_nparts(max_blocks, block_size);
   p.scale_log2 = scale * kLog2e;
-  p.part_o = nullptr;
-  p.part_ml = nullptr;
-  if (p.nparts > 1) {
-    const size_t need =
-        tlf_paged_decode_attn_workspace_bytes(batch, num_q_heads, head_dim, max_blocks, block_size);
-    if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 255u))
-      return TLF_E_WORKSPACE;
-    const size_t slots = static_cast<size_t>(batch) * p.nparts * num_q_heads;
-    p.part_o = static_cast<float *>(workspace);
-    p.part_ml = p.part_o + slots * kDh;
-  }
+  unsigned char *ws = static_cast<unsigned char *>(workspace);
+  const size_t slots = static_cast<size_t>(kMaxGrid) + batch;
+  p.meta = reinterpret_cast<int32_t *>(ws);
+  p.part_ml = reinterpret_cast<float *>(ws + decode_meta_bytes());
+  p.part_o = p.part_ml + slots * num_q_heads * 2;
+
+  // persistent grid: two workgroups per CU, fewer when the largest possible job is small
+  const int64_t max_tiles = static_cast<int64_t>(batch) * ((static_cast<int64_t>(max_blocks) * block_size + kTile - 1) / kTile);
+  int64_t grid = 2ll * device_cu_count();
+  if (grid > kMaxGrid) grid = kMaxGrid;
+  const int64_t by_work = (max_tiles + kMinTiles - 1) / kMinTiles;
+  if (grid > by_work) grid = by_work;
+  if (grid < 1) grid = 1;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const dim3 grid(p.nparts, batch);
+  const dim3 g(static_cast<unsigned>(grid));
+  const bool f8 = kv_dtype == TLF_KV_FP8_E4M3;
+#define TLF_DECODE(NW)                                                                         \
+  if (f8)                                                                                      \
+    hipLaunchKernelGGL((paged_decode_kernel<NW, true>), g, dim3(NW * 64), 0, s, p);            \
+  else                                                                                         \
+    hipLaunchKernelGGL((paged_decode_kernel<NW, false>), g, dim3(NW * 64), 0, s, p)
   switch (num_kv_heads) {
-    case 1: hipLaunchKernelGGL(paged_decode_kernel<1>, grid, dim3(64), 0, s, p); break;
-    case 2: hipLaunchKernelGGL(paged_decode_kernel<2>, grid, dim3(128), 0, s, p); break;
-    case 4: hipLaunchKernelGGL(paged_decode_kernel<4>, grid, dim3(256), 0, s, p); break;
-    case 8: hipLaunchKernelGGL(paged_decode_kernel<8>, grid, dim3(512), 0, s, p); break;
-    case 16: hipLaunchKernelGGL(paged_decode_kernel<16>, grid, dim3(1024), 0, s, p); break;
+    case 1: TLF_DECODE(1); break;
+    case 2: TLF_DECODE(2); break;
+    case 4: TLF_DECODE(4); break;
+    case 8: TLF_DECODE(8); break;
+    case 16: TLF_DECODE(16); break;
     default: return TLF_E_UNSUPPORTED;
   }
+#undef TLF_DECODE
   int rc = launch_status();
   if (rc != TLF_OK) return rc;
-  if (p.nparts > 1) {
-    hipLaunchKernelGGL(paged_decode_combine_kernel, dim3(num_q_heads, batch), dim3(64), 0, s, p);
-    rc = launch_status();
-  }
-  return rc;
+  hipLaunchKernelGGL(paged_decode_merge_kernel, dim3((num_q_heads + 7) / 8, batch), dim3(256), 0, s, p);
+  return launch_status();
 }

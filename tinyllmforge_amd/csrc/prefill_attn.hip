@@ -1,2 +1,353 @@
+// Varlen causal prefill attention for gfx950 (reference: the prefill branch of
+// tinyvllm/layers/attention.py:96-105, flash_attn_varlen_func with causal=True,
+// optionally reading K/V from the paged cache through block tables).
+//
+// MFMA-bound flash-style kernel.  A workgroup owns one sequence, one KV head and
+// a tile of query rows, and serves ALL Hq/Hkv query heads of that KV head, so a
+// K/V tile staged in LDS is reused by every head of the group.  The (row, head)
+// pairs of the tile are flattened into 64*CT "units"; a wave owns CT column
+// tiles of 16 units.
+//
+// Per 64-token K/V tile (global -> registers one tile ahead -> LDS, row-major):
+//   S^T[token, unit] = K . Q^T          v_mfma_f32_16x16x32_bf16, Q fragments in registers
+//   online softmax in fp32; causal mask bottom-right aligned
+//   O^T[dim, unit]  += V^T . P^T        v_mfma_f32_16x16x32_bf16; the V^T operand comes
+//                                       straight from the row-major tile with
+//                                       ds_read_b64_tr_b16 (LDS transpose read)
+// The rows of the K operand are permuted so that the S^T accumulator layout of
+// two 16-token sub-tiles is exactly the 32-token B operand of the second product:
+// P never leaves registers.  P is fed as a bf16 hi + lo pair.
 #include "common.h"
-extern "C" int tlf_varlen_prefill_attn(const void *, int64_t, const void *, int64_t, const void *, int64_t, int32_t, const float *, const float *, const int32_t *, const int32_t *, const int32_t *, int64_t, void *, int32_t, int32_t, int32_t, int32_t, int32_t, int32_t, int64_t, float, void *) { return TLF_E_UNSUPPORTED; }
+
+namespace tlf {
+
+constexpr int kPDh = 128;
+constexpr int kBKV = 64;            // K/V tokens per LDS tile
+constexpr int kPRow = kPDh + 8;     // padded LDS row (elements)
+constexpr float kPLog2e = 1.4426950408889634f;
+
+struct PrefillParams {
+  const unsigned short *q;
+  int64_t q_stride;
+  const unsigned char *k;
+  const unsigned char *v;
+  int64_t k_stride, v_stride;  // elements, packed layout only
+  const float *k_scale;
+  const float *v_scale;
+  const int32_t *cu_q;
+  const int32_t *cu_k;
+  const int32_t *block_tables;  // NULL: packed K/V
+  int64_t bt_stride;
+  unsigned short *out;
+  int32_t num_q_heads, num_kv_heads;
+  int32_t block_size;
+  int64_t num_cache_blocks;
+  float scale_log2;
+};
+
+// LDS transpose read: within each group of 16 lanes, lane i receives
+// {row0[i], row1[i], row2[i], row3[i]} where row j is the 16 elements addressed
+// (4 each) by lanes 4j .. 4j+3 of the group.
+__device__ __forceinline__ shortx4 lds_read_tr16(const unsigned short *p) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+      (shortx4 __attribute__((address_space(3))) *)(p));
+}
+
+__device__ __forceinline__ void fp8x16_to_bf16(const uint4 &in, uint4 &lo, uint4 &hi) {
+  auto cv = [](unsigned int w, unsigned int &a, unsigned int &b) {
+    const auto f0 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w), false);
+    const auto f1 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w), true);
+    a = pack_bf16x2(f0[0], f0[1]);
+    b = pack_bf16x2(f1[0], f1[1]);
+  };
+  cv(in.x, lo.x, lo.y);
+  cv(in.y, lo.z, lo.w);
+  cv(in.z, hi.x, hi.y);
+  cv(in.w, hi.z, hi.w);
+}
+
+template <int CT, bool KV8>
+__global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p) {
+  __shared__ __attribute__((aligned(16))) unsigned short Ks[kBKV][kPRow];
+  __shared__ __attribute__((aligned(16))) unsigned short Vs[kBKV][kPRow];
+  const int seq = blockIdx.z;
+  const int h = blockIdx.y;
+  const int group = p.num_q_heads / p.num_kv_heads;
+  const int bq = (64 * CT) / group;  // query rows per workgroup
+  const int row0 = blockIdx.x * bq;
+  const int q_begin = p.cu_q[seq];
+  const int lq = p.cu_q[seq + 1] - q_begin;
+  if (row0 >= lq) return;
+  const int k_begin = p.cu_k[seq];
+  const int lk = p.cu_k[seq + 1] - k_begin;
+  const int shift = lk - lq;  // cached prefix length: query i sees keys 0 .. shift + i
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int n = lane & 15, g = lane >> 4;
+
+  // units of this lane: u = wave*CT*16 + c*16 + n -> (row, head)
+  int urow[CT];
+  bool uok[CT];
+  bf16x8 qf[CT][4];
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    const int u = wave * CT * 16 + c * 16 + n;
+    urow[c] = row0 + u / group;
+    const int head = h * group + u % group;
+    uok[c] = urow[c] < lq;
+    const unsigned short *qp =
+        p.q + static_cast<int64_t>(q_begin + urow[c]) * p.q_stride + static_cast<int64_t>(head) * kPDh;
+#pragma unroll
+    for (int kc = 0; kc < 4; ++kc) {
+      Pack16 t;
+      t.u = make_uint4(0, 0, 0, 0);
+      if (uok[c]) t.u = *reinterpret_cast<const uint4 *>(qp + kc * 32 + g * 8);
+      qf[c][kc] = t.v;
+    }
+  }
+
+  const int last_row = min(row0 + bq, lq) - 1;
+  const int kv_end = min(lk, shift + last_row + 1);
+  const int32_t *bt = p.block_tables ? p.block_tables + seq * p.bt_stride : nullptr;
+  // e4m3 rows are dequantised as float(c) * scale[h]: the K scale is a constant factor of the scores
+  const float scale_log2 = p.scale_log2 * (KV8 ? p.k_scale[h] : 1.0f);
+  const int64_t cache_row = static_cast<int64_t>(p.num_kv_heads) * kPDh;
+
+  // K/V tile loader: bf16 rows are 16 chunks of 16 B, e4m3 rows 8 chunks of 16 B.
+  constexpr int kChunks = KV8 ? 8 : 16;
+  constexpr int kPasses = kBKV * kChunks / 256;
+  uint4 kreg[kPasses], vreg[kPasses];
+  auto load_tile = [&](int kv0) {
+#pragma unroll
+    for (int i = 0; i < kPasses; ++i) {
+      const int t = i * (256 / kChunks) + tid / kChunks;
+      const int ch = tid % kChunks;
+      const int tk = kv0 + t;
+      kreg[i] = make_uint4(0, 0, 0, 0);
+      vreg[i] = make_uint4(0, 0, 0, 0);
+      if (tk < kv_end) {
+        if (bt == nullptr) {
+          const int64_t ko = (static_cast<int64_t>(k_begin + tk) * p.k_stride + h * kPDh + ch * 8) * 2;
+          const int64_t vo = (static_cast<int64_t>(k_begin + tk) * p.v_stride + h * kPDh + ch * 8) * 2;
+          kreg[i] = *reinterpret_cast<const uint4 *>(p.k + ko);
+          vreg[i] = *reinterpret_cast<const uint4 *>(p.v + vo);
+        } else {
+          const int64_t blk = bt[tk / p.block_size];
+          if (blk >= 0 && blk < p.num_cache_blocks) {
+            const int64_t e = (blk * p.block_size + tk % p.block_size) * cache_row + h * kPDh;
+            const int64_t o = KV8 ? e + ch * 16 : (e + ch * 8) * 2;
+            kreg[i] = *reinterpret_cast<const uint4 *>(p.k + o);
+            vreg[i] = *reinterpret_cast<const uint4 *>(p.v + o);
+          }
+        }
+      }
+    }
+  };
+  auto store_tile = [&]() {
+#pragma unroll
+    for (int i = 0; i < kPasses; ++i) {
+      const int t = i * (256 / kChunks) + tid / kChunks;
+      const int ch = tid % kChunks;
+      if (KV8) {
+        uint4 lo, hi;
+        fp8x16_to_bf16(kreg[i], lo, hi);
+        *reinterpret_cast<uint4 *>(&Ks[t][ch * 16]) = lo;
+        *reinterpret_cast<uint4 *>(&Ks[t][ch * 16 + 8]) = hi;
+        fp8x16_to_bf16(vreg[i], lo, hi);
+        *reinterpret_cast<uint4 *>(&Vs[t][ch * 16]) = lo;
+        *reinterpret_cast<uint4 *>(&Vs[t][ch * 16 + 8]) = hi;
+      } else {
+        *reinterpret_cast<uint4 *>(&Ks[t][ch * 8]) = kreg[i];
+        *reinterpret_cast<uint4 *>(&Vs[t][ch * 8]) = vreg[i];
+      }
+    }
+  };
+
+  floatx4 acc[CT][8];
+  float m_run[CT], l_run[CT];
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    m_run[c] = -INFINITY;
+    l_run[c] = 0.f;
+#pragma unroll
+    for (int d = 0; d < 8; ++d) acc[c][d] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  load_tile(0);
+  store_tile();
+  __syncthreads();
+  for (int kv0 = 0; kv0 < kv_end; kv0 += kBKV) {
+    const bool more = kv0 + kBKV < kv_end;
+    if (more) load_tile(kv0 + kBKV);
+    // tiles that end at or before the first row's limit and inside lk need no mask
+    const bool need_mask = (kv0 + kBKV - 1 > shift + row0) || (kv0 + kBKV > lk);
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      if (kv0 + hh * 32 >= kv_end) break;  // uniform
+      // S^T for two 16-token sub-tiles; A row m of sub-tile s <-> token hh*32 + (m/4)*8 + s*4 + m%4
+      floatx4 s0[CT], s1[CT];
+#pragma unroll
+      for (int c = 0; c < CT; ++c) {
+        s0[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+        s1[c] = floatx4{0.f, 0.f, 0.f, 0.f};
+      }
+      const int tr0 = hh * 32 + (n >> 2) * 8 + (n & 3);
+#pragma unroll
+      for (int kc = 0; kc < 4; ++kc) {
+        Pack16 a0, a1;
+        a0.u = *reinterpret_cast<const uint4 *>(&Ks[tr0][kc * 32 + g * 8]);
+        a1.u = *reinterpret_cast<const uint4 *>(&Ks[tr0 + 4][kc * 32 + g * 8]);
+#pragma unroll
+        for (int c = 0; c < CT; ++c) {
+          s0[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0.v, qf[c][kc], s0[c], 0, 0, 0);
+          s1[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1.v, qf[c][kc], s1[c], 0, 0, 0);
+        }
+      }
+      // lane (n, g) of column tile c holds tokens kv0 + hh*32 + g*8 + j, j = 0..7
+      bf16x8 ph[CT], pl[CT];
+#pragma unroll
+      for (int c = 0; c < CT; ++c) {
+        float sv[8];
+        const int tbase = kv0 + hh * 32 + g * 8;
+        const int limit = min(shift + urow[c], lk - 1);  // last visible key of this unit
+        float mt = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float raw = (j < 4 ? s0[c][j] : s1[c][j - 4]) * scale_log2;
+          sv[j] = (!need_mask || tbase + j <= limit) ? raw : -INFINITY;
+          mt = fmaxf(mt, sv[j]);
+        }
+        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        const float m_new = fmaxf(m_run[c], mt);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = exp2f(m_run[c] - m_use);
+        float psum = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float pv = exp2f(sv[j] - m_use);
+          psum += pv;
+          ph[c][j] = static_cast<__bf16>(pv);
+          pl[c][j] = static_cast<__bf16>(pv - static_cast<float>(ph[c][j]));
+        }
+        l_run[c] = l_run[c] * alpha + psum;
+        m_run[c] = m_new;
+        if (alpha != 1.0f) {
+#pragma unroll
+          for (int d = 0; d < 8; ++d)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[c][d][i] *= alpha;
+        }
+      }
+      // O^T += V^T . P^T ; V^T fragment: lane (dim = d*16 + n, g) <- tokens hh*32 + g*8 + 0..7
+      const int vt = hh * 32 + g * 8 + (n >> 2);
+#pragma unroll
+      for (int d = 0; d < 8; ++d) {
+        const shortx4 v0 = lds_read_tr16(&Vs[vt][d * 16 + (n & 3) * 4]);
+        const shortx4 v1 = lds_read_tr16(&Vs[vt + 4][d * 16 + (n & 3) * 4]);
+        Pack16 vf;
+        vf.u = make_uint4(__builtin_bit_cast(uint2, v0).x, __builtin_bit_cast(uint2, v0).y,
+                          __builtin_bit_cast(uint2, v1).x, __builtin_bit_cast(uint2, v1).y);
+#pragma unroll
+        for (int c = 0; c < CT; ++c) {
+          acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, ph[c], acc[c][d], 0, 0, 0);
+          acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pl[c], acc[c][d], 0, 0, 0);
+        }
+      }
+    }
+    __syncthreads();
+    if (more) {
+      store_tile();
+      __syncthreads();
+    }
+  }
+
+  const float vscale = KV8 ? p.v_scale[h] : 1.0f;
+#pragma unroll
+  for (int c = 0; c < CT; ++c) {
+    float l = l_run[c];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (!uok[c]) continue;
+    const int u = wave * CT * 16 + c * 16 + n;
+    const int head = h * group + u % group;
+    const float inv = l > 0.f ? vscale / l : 0.f;
+    unsigned short *o = p.out + (static_cast<int64_t>(q_begin + urow[c]) * p.num_q_heads + head) * kPDh;
+#pragma unroll
+    for (int d = 0; d < 8; ++d) {
+      uint2 st;
+      st.x = pack_bf16x2(acc[c][d][0] * inv, acc[c][d][1] * inv);
+      st.y = pack_bf16x2(acc[c][d][2] * inv, acc[c][d][3] * inv);
+      *reinterpret_cast<uint2 *>(o + d * 16 + g * 4) = st;
+    }
+  }
+}
+
+}  // namespace tlf
+
+using namespace tlf;
+
+extern "C" int tlf_varlen_prefill_attn(const void *q, int64_t q_stride, const void *k,
+                                       int64_t k_stride, const void *v, int64_t v_stride,
+                                       int32_t kv_dtype, const float *k_scale, const float *v_scale,
+                                       const int32_t *cu_seqlens_q, const int32_t *cu_seqlens_k,
+                                       const int32_t *block_tables, int64_t block_table_stride,
+                                       void *out, int32_t num_seqs, int32_t max_seqlen_q,
+                                       int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim,
+                                       int32_t block_size, int64_t num_cache_blocks, float scale,
+                                       void *stream) {
+  if (num_seqs == 0 || max_seqlen_q == 0) return TLF_OK;
+  if (!q || !k || !v || !cu_seqlens_q || !cu_seqlens_k || !out) return TLF_E_NULL;
+  if (head_dim != kPDh) return TLF_E_UNSUPPORTED;
+  if (num_seqs < 0 || max_seqlen_q < 0 || num_q_heads <= 0 || num_kv_heads <= 0) return TLF_E_SHAPE;
+  if (num_q_heads % num_kv_heads) return TLF_E_SHAPE;
+  const int group = num_q_heads / num_kv_heads;
+  if (group != 1 && group != 2 && group != 4 && group != 8 && group != 16) return TLF_E_UNSUPPORTED;
+  if (q_stride < static_cast<int64_t>(num_q_heads) * head_dim || q_stride % 8) return TLF_E_SHAPE;
+  const bool paged = block_tables != nullptr;
+  if (paged) {
+    if (block_size <= 0 || num_cache_blocks <= 0 || block_table_stride <= 0) return TLF_E_SHAPE;
+    if (kv_dtype == TLF_KV_FP8_E4M3) {
+      if (!k_scale || !v_scale) return TLF_E_NULL;
+    } else if (kv_dtype != TLF_KV_BF16) {
+      return TLF_E_UNSUPPORTED;
+    }
+  } else {
+    if (kv_dtype != TLF_KV_BF16) return TLF_E_UNSUPPORTED;
+    if (k_stride < static_cast<int64_t>(num_kv_heads) * head_dim || k_stride % 8 ||
+        v_stride < static_cast<int64_t>(num_kv_heads) * head_dim || v_stride % 8)
+      return TLF_E_SHAPE;
+  }
+  if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(out)) return TLF_E_ALIGN;
+
+  PrefillParams p;
+  p.q = static_cast<const unsigned short *>(q);
+  p.q_stride = q_stride;
+  p.k = static_cast<const unsigned char *>(k);
+  p.v = static_cast<const unsigned char *>(v);
+  p.k_stride = k_stride;
+  p.v_stride = v_stride;
+  p.k_scale = k_scale;
+  p.v_scale = v_scale;
+  p.cu_q = cu_seqlens_q;
+  p.cu_k = cu_seqlens_k;
+  p.block_tables = block_tables;
+  p.bt_stride = block_table_stride;
+  p.out = static_cast<unsigned short *>(out);
+  p.num_q_heads = num_q_heads;
+  p.num_kv_heads = num_kv_heads;
+  p.block_size = block_size;
+  p.num_cache_blocks = num_cache_blocks;
+  p.scale_log2 = scale * kPLog2e;
+  constexpr int CT = 2;
+  const int bq = (64 * CT) / group;
+  const dim3 grid((max_seqlen_q + bq - 1) / bq, num_kv_heads, num_seqs);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (paged && kv_dtype == TLF_KV_FP8_E4M3) {
+    // the K scale is a per-head constant of the scores: fold it in on the device side per head
+    hipLaunchKernelGGL((prefill_attn_kernel<CT, true>), grid, dim3(256), 0, s, p);
+  } else {
+    hipLaunchKernelGGL((prefill_attn_kernel<CT, false>), grid, dim3(256), 0, s, p);
+  }
+  return launch_status();
+}

@@ -27,14 +27,19 @@ def _need(t: torch.Tensor, dtype, name: str):
 
 
 _workspaces: dict = {}
+_retired: list = []   # outgrown buffers stay alive: a captured graph may still point at them
 
 
-def _workspace(nbytes: int, device, tag: str) -> torch.Tensor:
-    """Grow-only scratch buffer per (device, tag, stream-capture state is the caller's concern)."""
+def _workspace(nbytes: int, device, tag: str, zero: bool = False) -> torch.Tensor:
+    """Grow-only scratch buffer per (device, tag).  Never freed, so pointers recorded in a
+    captured graph stay valid; ``zero`` buffers start zero-filled (decode arrival counters)."""
     key = (device, tag)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+        if ws is not None:
+            _retired.append(ws)
+        alloc = torch.zeros if zero else torch.empty
+        ws = alloc(max(nbytes, 256), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
 
@@ -230,7 +235,8 @@ def paged_decode_attention(q, k_cache, v_cache, context_lens, block_tables, scal
     assert k_cache.is_contiguous() and v_cache.is_contiguous() and block_tables.stride(1) == 1
     maxb = block_tables.shape[1]
     out = torch.empty(B, Hq * Dh, dtype=BF16, device=q.device)
-    nbytes = lib.tlf_paged_decode_attn_workspace_bytes(B, Hq, Dh, maxb, bs)
+    # sized for the largest batch so that one buffer serves every call (graph capture keeps its pointer)
+    nbytes = lib.tlf_paged_decode_attn_workspace_bytes(max(B, 1024), Hq, Dh, maxb, bs)
     ws = _workspace(nbytes, q.device, "decode")
     check(lib.tlf_paged_decode_attn(
         q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), kv_dtype_code(k_cache),
