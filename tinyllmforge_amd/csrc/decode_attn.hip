@@ -33,6 +33,8 @@
 // softmax statistics of a head live in the lanes that hold its O^T columns.
 // P is fed as a bf16 hi + lo pair (two MFMAs): matrix-core time is free in a
 // bandwidth-bound kernel and it removes the bf16 rounding of the probabilities.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace tlf {
@@ -98,8 +100,11 @@ struct TileRegs {
   bool ok;  // the tile's block-table entry names a real cache block
 };
 
-template <int NW, bool KV8>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4))) void paged_decode_kernel(const DecodeParams p) {
+// PF = tiles in flight per wave (register prefetch depth).  PF == 1 fits 128 VGPRs, i.e. two
+// 8-wave workgroups per CU; deeper prefetch runs one workgroup per CU with up to 256 VGPRs.
+template <int NW, bool KV8, int PF>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(PF == 1 ? 4 : 2, 4)))
+void paged_decode_kernel(const DecodeParams p) {
   constexpr int kThreads = NW * 64;
   __shared__ __attribute__((aligned(16))) unsigned short lds[NW][2][kTile][kLdsRow];
   __shared__ int s_prefix[kMaxBatch + 1];  // tiles before sequence b
@@ -247,63 +252,79 @@ __global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(4, 4)))
     float m_run = -INFINITY;  // running max (log2 domain), identical in the 4 lanes of a head
     float l_run = 0.f;        // this lane's share of the running sum
 
-    TileRegs<KV8> regs;
-    load_tile(t_begin, bt[t_begin / p.block_size], regs);
-    // block-table entry of the tile after this one (clamped to the segment: never read beyond it)
-    int next_blk = bt[min(t_begin + kTile, t_end - 1) / p.block_size];
-    for (int t0 = t_begin; t0 < t_end; t0 += kTile) {
-      wave_lds_fence();  // previous tile's LDS reads are done
-      store_tile(regs);
-      wave_lds_fence();
-      const bool tile_ok = regs.ok;
-      if (t0 + kTile < t_end) {
-        load_tile(t0 + kTile, next_blk, regs);
-        next_blk = bt[min(t0 + 2 * kTile, t_end - 1) / p.block_size];
-      }
+    // PF tiles are kept in flight: tile j of a group of PF lives in regs[j]; block-table entries
+    // are fetched PF tiles before the loads that need them.
+    TileRegs<KV8> regs[PF];
+    int next_blk[PF];
+#pragma unroll
+    for (int j = 0; j < PF; ++j) {
+      const int tj = t_begin + j * kTile;
+      if (tj < t_end) load_tile(tj, bt[tj / p.block_size], regs[j]);
+      next_blk[j] = bt[min(tj + PF * kTile, t_end - 1) / p.block_size];
+    }
+    for (int tg = t_begin; tg < t_end; tg += PF * kTile) {
+#pragma unroll
+      for (int j = 0; j < PF; ++j) {
+        const int t0 = tg + j * kTile;
+        if (t0 >= t_end) break;  // uniform
+        wave_lds_fence();  // previous tile's LDS reads are done
+        store_tile(regs[j]);
+        wave_lds_fence();
+        const bool tile_ok = regs[j].ok;
+        const int tn = t0 + PF * kTile;
+        if (tn < t_end) {
+          load_tile(tn, next_blk[j], regs[j]);
+          next_blk[j] = bt[min(tn + PF * kTile, t_end - 1) / p.block_size];
+        }
 
-      // S^T = K . Q^T : lane (n, g) gets tokens g*4 + i of head n
-      floatx4 s = floatx4{0.f, 0.f, 0.f, 0.f};
+        // S^T = K . Q^T : lane (n, g) gets tokens g*4 + i of head n
+        floatx4 s = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        Pack16 a;
-        a.u = *reinterpret_cast<const uint4 *>(&Ks[n][c * 32 + g * 8]);
-        s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[c], s, 0, 0, 0);
-      }
-      float sv[4];
-      float mt = -INFINITY;
+        for (int c = 0; c < 4; ++c) {
+          Pack16 a;
+          a.u = *reinterpret_cast<const uint4 *>(&Ks[n][c * 32 + g * 8]);
+          s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[c], s, 0, 0, 0);
+        }
+        float sv[4];
+        float mt = -INFINITY;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const bool valid = tile_ok && (t0 + g * 4 + i) < t_end;
-        sv[i] = valid ? s[i] * scale_log2 : -INFINITY;
-        mt = fmaxf(mt, sv[i]);
-      }
-      mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-      mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-      const float m_new = fmaxf(m_run, mt);
-      // -inf only while every token so far sat in a skipped block: keep the exponents finite
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = exp2f(m_run - m_use);
-      float psum = 0.f;
-      bf16x4 pb, pl;
+        for (int i = 0; i < 4; ++i) {
+          const bool valid = tile_ok && (t0 + g * 4 + i) < t_end;
+          sv[i] = valid ? s[i] * scale_log2 : -INFINITY;
+          mt = fmaxf(mt, sv[i]);
+        }
+        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
+        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        const float m_new = fmaxf(m_run, mt);
+        // -inf only while every token so far sat in a skipped block: keep the exponents finite
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = exp2f(m_run - m_use);
+        float psum = 0.f;
+        bf16x4 pb, pl;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float pv = exp2f(sv[i] - m_use);
-        psum += pv;
-        pb[i] = static_cast<__bf16>(pv);
-        pl[i] = static_cast<__bf16>(pv - static_cast<float>(pb[i]));
-      }
-      l_run = l_run * alpha + psum;
-      m_run = m_new;
-      const shortx4 pbs = __builtin_bit_cast(shortx4, pb);
-      const shortx4 pls = __builtin_bit_cast(shortx4, pl);
+        for (int i = 0; i < 4; ++i) {
+          const float pv = exp2f(sv[i] - m_use);
+          psum += pv;
+          pb[i] = static_cast<__bf16>(pv);
+          pl[i] = static_cast<__bf16>(pv - static_cast<float>(pb[i]));
+        }
+        l_run = l_run * alpha + psum;
+        m_run = m_new;
+        const shortx4 pbs = __builtin_bit_cast(shortx4, pb);
+        const shortx4 pls = __builtin_bit_cast(shortx4, pl);
+        // the running max rarely moves after the first tiles: skip the 32 multiplies then (wave-uniform)
+        const bool rescale = __any(alpha != 1.0f);
 #pragma unroll
-      for (int d = 0; d < 8; ++d) {
-        // A = V^T fragment: lane (dim = d*16 + n, g) <- tokens g*4 + 0..3 (transpose read)
-        const shortx4 vf = lds_read_tr16_b64(&Vs[g * 4 + (n >> 2)][d * 16 + (n & 3) * 4]);
+        for (int d = 0; d < 8; ++d) {
+          // A = V^T fragment: lane (dim = d*16 + n, g) <- tokens g*4 + 0..3 (transpose read)
+          const shortx4 vf = lds_read_tr16_b64(&Vs[g * 4 + (n >> 2)][d * 16 + (n & 3) * 4]);
+          if (rescale) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) acc[d][i] *= alpha;
-        acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pbs, acc[d], 0, 0, 0);
-        acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pls, acc[d], 0, 0, 0);
+            for (int i = 0; i < 4; ++i) acc[d][i] *= alpha;
+          }
+          acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pbs, acc[d], 0, 0, 0);
+          acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pls, acc[d], 0, 0, 0);
+        }
       }
     }
     l_run += __shfl_xor(l_run, 16, 64);
@@ -408,6 +429,34 @@ inline int device_cu_count() {
   return cus;
 }
 
+// Workgroups per CU of the persistent grid.  Measured on MI355X (config: B=64, ctx 512..4096):
+// 1 -> 109 us, 2 -> 116 us, 3 -> 119 us, 4 -> 125 us per call: fewer, longer shares mean fewer
+// partials and less contention.  TLF_DECODE_WGS_PER_CU overrides for tuning (2 and more need
+// TLF_DECODE_PREFETCH=1 to fit the register file).
+inline int decode_wgs_per_cu() {
+  static int v = 0;
+  if (v == 0) {
+    v = 1;
+    if (const char *e = getenv("TLF_DECODE_WGS_PER_CU")) {
+      const int x = atoi(e);
+      if (x >= 1 && x <= 4) v = x;
+    }
+  }
+  return v;
+}
+
+inline int decode_prefetch() {
+  static int v = 0;
+  if (v == 0) {
+    v = 1;  // measured on MI355X: depth 2 and 3 are no faster (the stream is not latency bound)
+    if (const char *e = getenv("TLF_DECODE_PREFETCH")) {
+      const int x = atoi(e);
+      if (x >= 1 && x <= 3) v = x;
+    }
+  }
+  return v;
+}
+
 inline size_t decode_meta_bytes() { return 2 * kMaxBatch * sizeof(int32_t); }
 
 }  // namespace tlf
@@ -480,7 +529,7 @@ extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void
 
   // persistent grid: two workgroups per CU, fewer when the largest possible job is small
   const int64_t max_tiles = static_cast<int64_t>(batch) * ((static_cast<int64_t>(max_blocks) * block_size + kTile - 1) / kTile);
-  int64_t grid = 2ll * device_cu_count();
+  int64_t grid = static_cast<int64_t>(decode_wgs_per_cu()) * device_cu_count();
   if (grid > kMaxGrid) grid = kMaxGrid;
   const int64_t by_work = (max_tiles + kMinTiles - 1) / kMinTiles;
   if (grid > by_work) grid = by_work;
@@ -488,11 +537,19 @@ extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 g(static_cast<unsigned>(grid));
   const bool f8 = kv_dtype == TLF_KV_FP8_E4M3;
-#define TLF_DECODE(NW)                                                                         \
-  if (f8)                                                                                      \
-    hipLaunchKernelGGL((paged_decode_kernel<NW, true>), g, dim3(NW * 64), 0, s, p);            \
-  else                                                                                         \
-    hipLaunchKernelGGL((paged_decode_kernel<NW, false>), g, dim3(NW * 64), 0, s, p)
+  const int pf = decode_prefetch();
+#define TLF_DECODE_PF(NW, F8, PF) \
+  hipLaunchKernelGGL((paged_decode_kernel<NW, F8, PF>), g, dim3(NW * 64), 0, s, p)
+#define TLF_DECODE(NW)                                        \
+  if (f8) {                                                   \
+    if (pf == 1) TLF_DECODE_PF(NW, true, 1);                  \
+    else if (pf == 2) TLF_DECODE_PF(NW, true, 2);             \
+    else TLF_DECODE_PF(NW, true, 3);                          \
+  } else {                                                    \
+    if (pf == 1) TLF_DECODE_PF(NW, false, 1);                 \
+    else if (pf == 2) TLF_DECODE_PF(NW, false, 2);            \
+    else TLF_DECODE_PF(NW, false, 3);                         \
+  }
   switch (num_kv_heads) {
     case 1: TLF_DECODE(1); break;
     case 2: TLF_DECODE(2); break;
@@ -502,6 +559,7 @@ extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void
     default: return TLF_E_UNSUPPORTED;
   }
 #undef TLF_DECODE
+#undef TLF_DECODE_PF
   int rc = launch_status();
   if (rc != TLF_OK) return rc;
   hipLaunchKernelGGL(paged_decode_merge_kernel, dim3((num_q_heads + 7) / 8, batch), dim3(256), 0, s, p);
