@@ -1,0 +1,126 @@
+"""CPU restatement of one Qwen3 decoder forward and of a greedy generate loop
+(test infrastructure: see ``oracle/__init__.py``).
+
+Follows the reference's op order (tinyvllm/models/qwen3.py:74-96, 123-130, 158-172, 185-195,
+229-234; layers/embed_head.py:58-63; layers/sampler.py:13-14) and its step inputs
+(engine/model_runner.py:164-228), including ``positions = len(seq)`` for decode steps
+(model_runner.py:219).
+
+Every linear is the exactly rounded one (``ops.linear_exact``: fp64 accumulation, one rounding
+to bf16) so that the token ids do not depend on the accumulation order of the host's BLAS;
+the reference's ``F.linear`` is the same contraction with an unspecified fp32 order.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import ops as O
+
+
+class OracleQwen3:
+    def __init__(self, cfg: dict, params: dict):
+        """``params``: ``{name: tensor}`` with the reference's packed parameter names
+        (``model.layers.N.self_attn.qkv_proj.weight`` ...)."""
+        self.cfg = dict(cfg)
+        self.p = {k: v.detach().cpu() for k, v in params.items()}
+        self.p64 = {k: v.double() for k, v in self.p.items() if k.endswith("proj.weight") or "embed_tokens" in k
+                    or k.startswith("lm_head")}
+        c = self.cfg
+        self.Hq, self.Hkv, self.Dh = c["num_attention_heads"], c["num_key_value_heads"], c["head_dim"]
+        self.eps = c.get("rms_norm_eps", 1e-6)
+        self.table = O.rope_table(self.Dh, c.get("max_position_embeddings", 40960), c.get("rope_theta", 1e6))
+        self.L = c["num_hidden_layers"]
+        if "lm_head.weight" not in self.p64:
+            self.p64["lm_head.weight"] = self.p64["model.embed_tokens.weight"]
+
+    def lin(self, x, name):
+        return (x.double() @ self.p64[name].t()).to(x.dtype)
+
+    def forward(self, input_ids, positions, caches, slot_mapping, attend):
+        """``caches[l] = (k_cache, v_cache)``; ``attend(q, k, v, k_cache, v_cache)`` does the step's attention."""
+        p = self.p
+        x = O.embedding(input_ids, p["model.embed_tokens.weight"])
+        residual = None
+        q_size, kv_size = self.Hq * self.Dh, self.Hkv * self.Dh
+        for l in range(self.L):
+            pre = f"model.layers.{l}."
+            if residual is None:
+                residual = x
+                x = O.rms_norm(x, p[pre + "input_layernorm.weight"], self.eps)
+            else:
+                x, residual = O.add_rms_norm(x, residual, p[pre + "input_layernorm.weight"], self.eps)
+            qkv = self.lin(x, pre + "self_attn.qkv_proj.weight")
+            q, k, v = qkv.split([q_size, kv_size, kv_size], dim=-1)
+            n = q.shape[0]
+            q = O.rms_norm(q.reshape(n, self.Hq, self.Dh), p[pre + "self_attn.q_norm.weight"], self.eps).reshape(n, -1)
+            k = O.rms_norm(k.reshape(n, self.Hkv, self.Dh), p[pre + "self_attn.k_norm.weight"], self.eps).reshape(n, -1)
+            q, k = O.rope(positions, q, k, self.table, self.Dh)
+            kc, vc = caches[l]
+            O.store_kvcache(k.view(n, self.Hkv, self.Dh), v.reshape(n, self.Hkv, self.Dh), kc, vc, slot_mapping)
+            o = attend(q.view(n, self.Hq, self.Dh), k.view(n, self.Hkv, self.Dh), v.reshape(n, self.Hkv, self.Dh), kc, vc)
+            x = self.lin(o, pre + "self_attn.o_proj.weight")
+            x, residual = O.add_rms_norm(x, residual, p[pre + "post_attention_layernorm.weight"], self.eps)
+            x = self.lin(x, pre + "mlp.gate_up_proj.weight")
+            x = O.silu_and_mul(x)
+            x = self.lin(x, pre + "mlp.down_proj.weight")
+        x, _ = O.add_rms_norm(x, residual, p["model.norm.weight"], self.eps)
+        return x
+
+    def logits(self, hidden):
+        return (hidden.double() @ self.p64["lm_head.weight"].t()).to(hidden.dtype)
+
+
+def greedy_generate(model: OracleQwen3, prompts: list[list[int]], max_tokens: int, block_size: int = 256,
+                    position_quirk: bool = True):
+    """All prompts prefilled in one step, then ``max_tokens - 1`` decode steps of the whole batch.
+
+    Returns ``(token_ids, margins, topk)``: the generated ids per sequence; per step and sequence the
+    gap between the two largest logits (fp32 of the bf16 logits), to judge near-ties; and per step
+    and sequence the four largest logits as ``(ids, values)``.
+    """
+    B = len(prompts)
+    Hkv, Dh = model.Hkv, model.Dh
+    max_len = max(len(p) for p in prompts) + max_tokens + 1
+    nblk_seq = -(-max_len // block_size)
+    caches = [(torch.zeros(B * nblk_seq, block_size, Hkv, Dh, dtype=torch.bfloat16),
+               torch.zeros(B * nblk_seq, block_size, Hkv, Dh, dtype=torch.bfloat16)) for _ in range(model.L)]
+    bt = torch.arange(B * nblk_seq, dtype=torch.int32).view(B, nblk_seq)     # sequence b owns blocks b*n .. b*n+n-1
+    scale = O.softmax_scale(Dh)
+    seqs = [list(p) for p in prompts]
+    out = [[] for _ in range(B)]
+    margins, topk = [], []
+
+    def slot(b, t):
+        return int(bt[b, t // block_size]) * block_size + t % block_size
+
+    def sample(hidden_rows):
+        lg = model.logits(hidden_rows)
+        top = lg.float().topk(4, dim=-1)
+        margins.append((top.values[:, 0] - top.values[:, 1]).tolist())
+        topk.append((top.indices.tolist(), top.values.tolist()))
+        return O.greedy_sample(lg).tolist()
+
+    # prefill
+    lens = [len(s) for s in seqs]
+    ids = torch.tensor([t for s in seqs for t in s], dtype=torch.int64)
+    pos = torch.tensor([t for s in seqs for t in range(len(s))], dtype=torch.int64)
+    slots = torch.tensor([slot(b, t) for b, s in enumerate(seqs) for t in range(len(s))], dtype=torch.int32)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32)
+    h = model.forward(ids, pos, caches, slots,
+                      lambda q, k, v, kc, vc: O.varlen_prefill_attention(q, k, v, cu, cu, scale))
+    toks = sample(h[(cu[1:] - 1).long()])
+    for b in range(B):
+        seqs[b].append(toks[b]); out[b].append(toks[b])
+    # decode
+    for _ in range(max_tokens - 1):
+        n = [len(s) for s in seqs]
+        ids = torch.tensor([s[-1] for s in seqs], dtype=torch.int64)
+        pos = torch.tensor([(x if position_quirk else x - 1) for x in n], dtype=torch.int64)
+        slots = torch.tensor([slot(b, n[b] - 1) for b in range(B)], dtype=torch.int32)
+        cl = torch.tensor(n, dtype=torch.int32)
+        h = model.forward(ids, pos, caches, slots,
+                          lambda q, k, v, kc, vc: O.paged_decode_attention(q, kc, vc, cl, bt, scale))
+        toks = sample(h)
+        for b in range(B):
+            seqs[b].append(toks[b]); out[b].append(toks[b])
+    return out, margins, topk

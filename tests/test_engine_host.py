@@ -1,0 +1,236 @@
+"""Host logic (CPU): sequence block math, block manager order and hashing, scheduler policy,
+and the integer inputs of the hot path (slot mapping, block tables, positions) - bit exact.
+
+Pins: closed forms on hand-built states (block boundaries len % 256 in {0, 1, 255}), the
+xxh64 library as known answer, and the invariants slot // bs == block_table[pos // bs],
+slot % bs == pos % bs.
+"""
+import numpy as np
+import pytest
+import xxhash
+
+from tinyllmforge_amd.config import Config, ModelConfig, QWEN3_SHAPES
+from tinyllmforge_amd.engine import inputs as I
+from tinyllmforge_amd.engine.block_manager import BlockManager
+from tinyllmforge_amd.engine.scheduler import Scheduler
+from tinyllmforge_amd.engine.sequence import Sequence, SequenceStatus
+from tinyllmforge_amd.sampling_params import SamplingParams
+
+BS = 256
+
+
+@pytest.fixture(autouse=True)
+def _bs():
+    Sequence.block_size = BS
+    yield
+
+
+def seq(n, start=0, **kw):
+    return Sequence(list(range(start, start + n)), SamplingParams(**kw) if kw else None)
+
+
+@pytest.mark.parametrize("n,blocks,last", [(1, 1, 1), (255, 1, 255), (256, 1, 256), (257, 2, 1), (512, 2, 256), (513, 3, 1)])
+def test_sequence_block_math(n, blocks, last):
+    s = seq(n)
+    assert (len(s), s.num_blocks, s.last_block_num_tokens) == (n, blocks, last)
+    assert s.block(blocks - 1) == list(range((blocks - 1) * BS, n))
+    s.append_token(7)
+    assert len(s) == n + 1 and s.last_token == 7 and s.num_completion_tokens == 1 and s.completion_token_ids == [7]
+
+
+def test_block_hash_known_answers():
+    assert xxhash.xxh64(b"").intdigest() == 0xEF46DB3751D8E999            # published xxh64 vector (seed 0)
+    toks = [5, 0, 2 ** 40, 9]
+    raw = np.array(toks, dtype=np.int64).tobytes()
+    assert len(raw) == 32 and raw[:8] == (5).to_bytes(8, "little")
+    assert BlockManager.compute_hash(toks) == xxhash.xxh64(raw).intdigest()
+    pre = 0x1234567890ABCDEF
+    assert BlockManager.compute_hash(toks, pre) == xxhash.xxh64(pre.to_bytes(8, "little") + raw).intdigest()
+    assert BlockManager.compute_hash(toks, pre) != BlockManager.compute_hash(toks)
+
+
+def test_block_manager_fifo_order_prefix_hits_and_revival():
+    bm = BlockManager(8, BS)
+    a = seq(600)                                     # 3 blocks: two full, one partial
+    assert bm.can_allocate(a)
+    bm.allocate(a)
+    assert a.block_table == [0, 1, 2] and a.num_cached_tokens == 0
+    assert bm.blocks[0].hash != -1 and bm.blocks[2].hash == -1        # only full blocks are hashed
+    b = Sequence(list(range(512)) + [9999] * 10)                      # shares two full blocks
+    bm.allocate(b)
+    assert b.block_table == [0, 1, 3] and b.num_cached_tokens == 512
+    assert bm.blocks[0].ref_count == 2
+    bm.deallocate(a)
+    assert list(bm.free_block_ids) == [4, 5, 6, 7, 2]                 # freed to the right, shared blocks stay
+    bm.deallocate(b)
+    assert list(bm.free_block_ids) == [4, 5, 6, 7, 2, 3, 1, 0]        # reversed table order
+    c = seq(300)                                                      # first block revived by its hash
+    bm.allocate(c)
+    assert c.block_table == [0, 4] and c.num_cached_tokens == 256
+    d = Sequence([1] + list(range(1, 600)))                           # first block differs: all fresh
+    bm.allocate(d)
+    assert d.num_cached_tokens == 0 and d.block_table == [5, 6, 7]
+
+
+def test_block_manager_full_hit_recomputes_last_block():
+    bm = BlockManager(4, BS)
+    a = seq(512)
+    bm.allocate(a)
+    b = seq(512)
+    bm.allocate(b)
+    assert b.block_table == [0, 1]
+    assert b.num_cached_tokens == 256           # never equal to len: at least the last block is prefilled
+
+
+def test_block_manager_append_protocol():
+    bm = BlockManager(4, BS)
+    s = seq(255)
+    bm.allocate(s)
+    s.append_token(1)                            # len 256: block becomes full on may_append
+    assert bm.can_append(s)
+    bm.may_append(s)
+    assert bm.blocks[s.block_table[-1]].hash == BlockManager.compute_hash(s.block(0))
+    s.append_token(2)                            # len 257: needs a new block
+    assert bm.can_append(s) == (len(bm.free_block_ids) >= 1)
+    bm.may_append(s)
+    assert s.block_table == [0, 1]
+    s.append_token(3)
+    bm.may_append(s)                             # nothing to do in the middle of a block
+    assert s.block_table == [0, 1]
+
+
+def _cfg(**kw):
+    base = dict(model=QWEN3_SHAPES["qwen3-0.6b"], num_kvcache_blocks=8, max_num_seqs=4, max_num_batched_tokens=4096,
+                max_model_len=2048)
+    base.update(kw)
+    return Config(**base)
+
+
+def test_scheduler_prefill_first_then_decode_and_finish():
+    sch = Scheduler(_cfg())
+    seqs = [seq(100, max_tokens=2, ignore_eos=True) for _ in range(3)]
+    for s in seqs:
+        sch.add(s)
+    batch, is_prefill = sch.schedule()
+    assert is_prefill and batch == seqs and all(s.status is SequenceStatus.RUNNING for s in seqs)
+    sch.postprocess(batch, [1, 2, 3])
+    batch, is_prefill = sch.schedule()
+    assert not is_prefill and batch == seqs
+    sch.postprocess(batch, [4, 5, 6])
+    assert sch.is_finished() and all(s.is_finished for s in seqs)
+    assert len(sch.block_manager.free_block_ids) == 8
+    assert seqs[1].completion_token_ids == [2, 5]
+
+
+def test_scheduler_token_budget_and_seq_limit():
+    sch = Scheduler(_cfg(max_num_batched_tokens=2048, max_num_seqs=2, num_kvcache_blocks=32))
+    for n in (1500, 600, 100):
+        sch.add(seq(n, max_tokens=1))
+    batch, _ = sch.schedule()
+    assert [len(s) for s in batch] == [1500]           # 1500 + 600 > 2048
+    sch.postprocess(batch, [0])
+    batch, _ = sch.schedule()
+    assert [len(s) for s in batch] == [600, 100]       # limited by max_num_seqs = 2
+
+
+def test_scheduler_preempts_newest_when_out_of_blocks():
+    sch = Scheduler(_cfg(num_kvcache_blocks=2))
+    a, b = seq(256, max_tokens=8, ignore_eos=True), seq(256, start=1000, max_tokens=8, ignore_eos=True)
+    sch.add(a); sch.add(b)
+    batch, is_prefill = sch.schedule()
+    assert is_prefill and len(batch) == 2
+    sch.postprocess(batch, [1, 1])                      # both at 257 tokens: each needs a new block, none free
+    batch, is_prefill = sch.schedule()
+    assert not is_prefill and batch == [a]              # b (newest) preempted, its block goes to a
+    assert b.status is SequenceStatus.WAITING and not b.block_table and sch.waiting[0] is b
+    assert a.block_table == [0, 1]
+
+
+def test_eos_stops_unless_ignored():
+    cfg = _cfg(); cfg.eos = 42
+    sch = Scheduler(cfg)
+    a, b = seq(10, max_tokens=5), seq(10, max_tokens=5, ignore_eos=True)
+    sch.add(a); sch.add(b)
+    batch, _ = sch.schedule()
+    sch.postprocess(batch, [42, 42])
+    assert a.is_finished and not b.is_finished
+
+
+# ----------------------------------------------------------------------------- integer inputs
+def test_prefill_inputs_closed_form_no_prefix():
+    bm = BlockManager(16, BS)
+    seqs = [seq(300), seq(256, start=5000), seq(1, start=9000)]
+    for s in seqs:
+        bm.allocate(s)
+    d = I.prefill_inputs(seqs, BS)
+    assert d["input_ids"].dtype == np.int64 and d["positions"].dtype == np.int64
+    assert d["slot_mapping"].dtype == np.int32 and d["cu_seqlens_q"].dtype == np.int32
+    assert d["cu_seqlens_q"].tolist() == [0, 300, 556, 557] == d["cu_seqlens_k"].tolist()
+    assert (d["max_seqlen_q"], d["max_seqlen_k"]) == (300, 300) and d["block_tables"] is None
+    assert d["input_ids"].tolist() == list(range(300)) + list(range(5000, 5256)) + [9000]
+    assert d["positions"].tolist() == list(range(300)) + list(range(256)) + [0]
+    # blocks were handed out in order 0,1 | 2 | 3
+    expect = list(range(0, 300)) + list(range(2 * 256, 3 * 256)) + [3 * 256]
+    assert d["slot_mapping"].tolist() == expect
+    # invariants: slot // bs is the table entry of the token's block, slot % bs its offset
+    off = 0
+    for s in seqs:
+        n = len(s)
+        sl = d["slot_mapping"][off:off + n]
+        t = np.arange(n)
+        assert (sl // BS == np.asarray(s.block_table)[t // BS]).all() and (sl % BS == t % BS).all()
+        off += n
+
+
+def test_prefill_inputs_with_prefix_hit():
+    bm = BlockManager(16, BS)
+    a = seq(700)
+    bm.allocate(a)
+    b = Sequence(list(range(512)) + [7] * 100)           # 512 cached tokens
+    bm.allocate(b)
+    c = seq(50, start=3000)
+    bm.allocate(c)
+    d = I.prefill_inputs([b, c], BS)
+    assert d["cu_seqlens_q"].tolist() == [0, 100, 150] and d["cu_seqlens_k"].tolist() == [0, 612, 662]
+    assert d["positions"].tolist() == list(range(512, 612)) + list(range(50))
+    assert d["input_ids"][:100].tolist() == [7] * 100
+    assert d["slot_mapping"].tolist() == [b.block_table[2] * BS + i for i in range(100)] + [c.block_table[0] * BS + i for i in range(50)]
+    assert d["block_tables"].tolist() == [b.block_table, c.block_table + [-1, -1]]
+    assert d["block_tables"].dtype == np.int32
+
+
+@pytest.mark.parametrize("n", [1, 255, 256, 257, 511, 512, 513])
+def test_decode_inputs_closed_form(n):
+    bm = BlockManager(16, BS)
+    s = seq(n)
+    bm.allocate(s)
+    other = seq(300, start=777)
+    bm.allocate(other)
+    for q in (s, other):
+        q.append_token(11)
+        bm.may_append(q)
+    d = I.decode_inputs([s, other], BS)
+    L = n + 1
+    assert d["input_ids"].tolist() == [11, 11]
+    assert d["positions"].tolist() == [L, 301]                      # the reference feeds len(seq), not len - 1
+    assert I.decode_inputs([s], BS, position_quirk=False)["positions"].tolist() == [L - 1]
+    assert d["context_lens"].tolist() == [L, 301]
+    t = L - 1                                                       # index of the fed token
+    assert d["slot_mapping"][0] == s.block_table[t // BS] * BS + t % BS
+    assert d["slot_mapping"][1] == other.block_table[300 // BS] * BS + 300 % BS
+    w = max(len(s.block_table), len(other.block_table))
+    assert d["block_tables"].shape == (2, w)
+    assert d["block_tables"][0, :len(s.block_table)].tolist() == s.block_table
+    assert (d["block_tables"][0, len(s.block_table):] == -1).all()
+
+
+def test_config_accepts_shape_names_and_dicts():
+    c = Config("qwen3-8b")
+    assert c.hf_config.hidden_size == 4096 and c.hf_config.head_dim == 128 and not c.hf_config.tie_word_embeddings
+    c2 = Config(dict(hidden_size=256, num_hidden_layers=2, num_attention_heads=2, num_key_value_heads=1,
+                     intermediate_size=512, max_position_embeddings=1024), max_model_len=4096, max_num_batched_tokens=4096)
+    assert c2.max_model_len == 1024 and c2.hf_config.head_dim == 128
+    with pytest.raises(AssertionError):
+        Config("qwen3-8b", kvcache_block_size=100)
+    with pytest.raises(AssertionError):
+        Config("qwen3-8b", tensor_parallel_size=2)

@@ -1,0 +1,173 @@
+"""GPU end-to-end parity: LLM.generate() on BASELINE config 1 against the oracle's golden ids,
+and engine-level behaviour (graph vs eager, fused vs unfused, prefix cache, preemption)."""
+import json
+import os
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "c1_greedy.json")
+
+
+def c1_prompts():
+    g = torch.Generator().manual_seed(0)
+    return torch.randint(0, 151936, (4, 128), generator=g).tolist()
+
+
+@pytest.fixture(scope="module")
+def golden():
+    with open(GOLDEN) as f:
+        return json.load(f)
+
+
+@pytest.fixture(scope="module")
+def llm_c1():
+    from tinyllmforge_amd import LLM
+    llm = LLM("qwen3-0.6b", max_model_len=1024, max_num_batched_tokens=4096, max_num_seqs=8,
+              num_kvcache_blocks=48, enforce_eager=False, seed=0)
+    yield llm
+    llm.exit()
+
+
+def ulp_of(v):
+    import math
+    return 2.0 ** (math.floor(math.log2(abs(v))) - 7) if v != 0 else 2.0 ** -133
+
+
+def near_tie(golden, step, s, ulps=1):
+    """The oracle's two best logits are within ``ulps`` bf16 ulp of each other (0 = exact tie)."""
+    top = golden["top4_logits"][step][s]
+    return (top[0] - top[1]) <= ulps * ulp_of(top[0])
+
+
+def test_c1_greedy_token_ids_free_running(llm_c1, golden):
+    """4 x 128 random prompt ids, 32 greedy tokens through LLM.generate() with hipGraph decode.
+
+    Ids must be bit-identical to the CPU oracle's up to each sequence's first step where the oracle's
+    own top-2 logits are within one bf16 ulp: there the choice is decided by the last bit of a
+    28-layer bf16 pipeline (accumulation order), which no two implementations share; the
+    teacher-forced test below covers every step after that point.
+    """
+    from tinyllmforge_amd import SamplingParams
+    prompts = c1_prompts()
+    assert [p[:4] for p in prompts] == golden["prompt_first_tokens"]
+    out = llm_c1.generate(prompts, SamplingParams(temperature=0.0, max_tokens=32, ignore_eos=True))
+    got = [o["token_ids"] for o in out]
+    assert all(len(g) == 32 for g in got)
+    exact = 0
+    for s in range(4):
+        safe = next((t for t in range(32) if near_tie(golden, t, s)), 32)
+        assert got[s][:safe] == golden["token_ids"][s][:safe], f"seq {s} differs before its first near-tie (step {safe})"
+        exact += got[s] == golden["token_ids"][s]
+    print(f"free-running: {exact} of 4 sequences identical over all 32 tokens")
+    st = llm_c1.last_stats
+    # like the reference (llm_engine.py:58) the prefill count is taken after the sampled token is appended
+    assert st["prefill_steps"] == 1 and st["prefill_tokens"] == 516 and st["decode_steps"] == 31
+
+
+def test_c1_teacher_forced_every_step(llm_c1, golden):
+    """Feed the oracle's tokens and check all 4 x 32 decisions and logits of the HIP path.
+
+    After 28 bf16 layers the logits of the two pipelines agree to within 3 bf16 ulp (measured: 2);
+    a decision is therefore required to be identical whenever the oracle's margin exceeds 2 ulp, and
+    must otherwise fall on one of the oracle's candidates inside that band.
+    """
+    from tinyllmforge_amd.engine.sequence import Sequence
+    from tinyllmforge_amd.sampling_params import SamplingParams
+    runner, sch = llm_c1.model_runner, llm_c1.scheduler
+    sp = SamplingParams(temperature=0.0, max_tokens=32, ignore_eos=True)
+    seqs0 = [Sequence(p, sp) for p in c1_prompts()]
+    for s in seqs0:
+        sch.add(s)
+    same, tied, worst = 0, 0, 0.0
+    for step in range(32):
+        seqs, is_prefill = sch.schedule()
+        assert [q.seq_id for q in seqs] == [q.seq_id for q in seqs0] and is_prefill == (step == 0)
+        ids, pos = runner.prepare_prefill(seqs) if is_prefill else runner.prepare_decode(seqs)
+        logits = runner.run_model(ids, pos, is_prefill).float().cpu()
+        from tinyllmforge_amd.utils.context import reset_context
+        reset_context()
+        choice = logits.argmax(-1).tolist()
+        for s in range(4):
+            want = golden["token_ids"][s][step]
+            cand, vals = golden["top4_ids"][step][s], golden["top4_logits"][step][s]
+            for c, v in zip(cand, vals):                       # logits of the oracle's best candidates agree
+                worst = max(worst, abs(logits[s, c].item() - v))
+                assert abs(logits[s, c].item() - v) <= 3 * ulp_of(v), (step, s, c, logits[s, c].item(), v)
+            if near_tie(golden, step, s, ulps=2):
+                allowed = [c for c, v in zip(cand, vals) if vals[0] - v <= 3 * ulp_of(vals[0])]
+                assert choice[s] in allowed, (step, s, choice[s], cand, vals)
+                tied += 1
+            else:
+                assert choice[s] == want, (step, s, choice[s], want, vals)
+            same += choice[s] == want
+        sch.postprocess(seqs, [golden["token_ids"][s][step] for s in range(4)])
+    assert sch.is_finished()
+    print(f"teacher-forced: {same}/128 decisions identical, {tied} near-tie steps, max |logit diff| {worst:.4f}")
+    assert same >= 128 - tied
+
+
+def test_c1_eager_equals_graph_and_rerun_hits_prefix_cache(llm_c1, golden):
+    from tinyllmforge_amd import SamplingParams
+    sp = SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True)
+    prompts = [p + p for p in c1_prompts()]                   # 256 tokens: one full (hashable) block each
+    a = [o["token_ids"] for o in llm_c1.generate(prompts, sp)]
+    runner = llm_c1.model_runner
+    runner.enforce_eager = True
+    try:
+        # second run: the first block of every prompt is a prefix-cache hit -> paged prefill path
+        b = [o["token_ids"] for o in llm_c1.generate(prompts, sp)]
+    finally:
+        runner.enforce_eager = False
+    assert llm_c1.last_stats["prefill_tokens"] == sum(len(p) + 1 for p in prompts)   # full lengths, counted after the append
+    assert a == b
+
+
+def test_unfused_layer_path_gives_identical_tokens(llm_c1):
+    from tinyllmforge_amd import SamplingParams
+    sp = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)
+    prompts = [p[:40] for p in c1_prompts()]
+    runner = llm_c1.model_runner
+    a = [o["token_ids"] for o in llm_c1.generate(prompts, sp)]
+    runner.enforce_eager = True
+    for layer in runner.model.model.layers:
+        layer.self_attn.fused = False
+    try:
+        b = [o["token_ids"] for o in llm_c1.generate(prompts, sp)]
+    finally:
+        runner.enforce_eager = False
+        for layer in runner.model.model.layers:
+            layer.self_attn.fused = True
+    assert a == b
+
+
+TINY = dict(hidden_size=256, num_hidden_layers=2, num_attention_heads=2, num_key_value_heads=1, head_dim=128,
+            intermediate_size=512, vocab_size=1024, max_position_embeddings=2048, tie_word_embeddings=True)
+
+
+def test_preemption_and_recompute_complete_every_request():
+    from tinyllmforge_amd import LLM, SamplingParams
+    llm = LLM(TINY, max_model_len=1024, max_num_batched_tokens=2048, max_num_seqs=4, num_kvcache_blocks=5,
+              enforce_eager=True, seed=1)
+    g = torch.Generator().manual_seed(3)
+    prompts = [torch.randint(0, 1024, (n,), generator=g).tolist() for n in (250, 255, 200, 256)]
+    out = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=20, ignore_eos=True))
+    assert [len(o["token_ids"]) for o in out] == [20] * 4
+    bm = llm.scheduler.block_manager
+    assert len(bm.free_block_ids) == 5 and not bm.used_block_ids
+    llm.exit()
+
+
+def test_temperature_sampling_runs_and_respects_greedy_rows():
+    from tinyllmforge_amd import LLM, SamplingParams
+    llm = LLM(TINY, max_model_len=512, max_num_batched_tokens=1024, max_num_seqs=4, num_kvcache_blocks=8,
+              enforce_eager=True, seed=1)
+    g = torch.Generator().manual_seed(4)
+    p = torch.randint(0, 1024, (30,), generator=g).tolist()
+    greedy = llm.generate([p], SamplingParams(temperature=0.0, max_tokens=5, ignore_eos=True))[0]["token_ids"]
+    mixed = llm.generate([p, p], [SamplingParams(temperature=0.0, max_tokens=5, ignore_eos=True),
+                                  SamplingParams(temperature=0.8, max_tokens=5, ignore_eos=True)])
+    assert mixed[0]["token_ids"] == greedy
+    assert all(0 <= t < 1024 for t in mixed[1]["token_ids"])
+    llm.exit()

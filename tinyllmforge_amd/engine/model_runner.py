@@ -1,0 +1,217 @@
+"""Host -> GPU boundary of one engine step (reference: tinyvllm/engine/model_runner.py:15-308).
+
+One process, one GPU: no process group, no shared-memory RPC.  Per step the runner builds the
+integer inputs on the host (``engine/inputs.py``), stages them in one pinned buffer, copies them
+to the device and runs the model either eagerly (prefill) or by replaying a captured hipGraph
+(decode; ``torch.cuda.CUDAGraph`` is the hipGraph wrapper on ROCm).  Graph padding rows carry
+slot -1 and context length 0, so they neither write the KV cache nor read it.
+"""
+from __future__ import annotations
+
+import numpy as np
+import torch
+
+from ..config import Config
+from ..layers.sampler import Sampler
+from ..models.qwen3 import Qwen3ForCausalLM
+from ..utils.context import get_context, reset_context, set_context
+from ..utils.loader import load_model, random_init_
+from . import inputs as I
+from .sequence import Sequence
+
+
+class ModelRunner:
+    def __init__(self, config: Config, rank: int = 0, event=None, state_dict: dict | None = None):
+        assert rank == 0
+        if not torch.cuda.is_available():
+            raise RuntimeError("ModelRunner needs a GPU: the HIP hot path has no CPU fallback")
+        self.config = config
+        hf = config.hf_config
+        self.block_size = config.kvcache_block_size
+        Sequence.block_size = self.block_size
+        self.enforce_eager = config.enforce_eager
+        self.device = torch.device("cuda", torch.cuda.current_device())
+        self.kv_dtype = torch.bfloat16 if config.kv_cache_dtype == "bf16" else torch.float8_e4m3fn
+
+        default_dtype = torch.get_default_dtype()
+        torch.set_default_dtype(hf.torch_dtype)
+        try:
+            with torch.device(self.device):
+                self.model = Qwen3ForCausalLM(hf)
+            # the RoPE table is built on the host (same bits as a CPU restatement), then moved
+            self.model.to(self.device)
+            if state_dict is not None:
+                from ..utils.loader import load_state_dict
+                load_state_dict(self.model, state_dict)
+            elif isinstance(config.model, str) and __import__("os").path.isdir(config.model):
+                load_model(self.model, config.model)
+            else:
+                big = hf.hidden_size >= 2048
+                random_init_(self.model, seed=config.seed, device_fill=big)
+            if config.quantization == "w8a16":
+                self.model.quantize_linears_()
+        finally:
+            torch.set_default_dtype(default_dtype)
+        self.model.eval()
+        self.sampler = Sampler()
+        self.graphs = {}
+        self.graph_bs = []
+        with torch.inference_mode():
+            self.warmup_model()
+            self.allocate_kv_cache()
+            if not self.enforce_eager:
+                self.capture_graphs()
+
+    def exit(self):
+        self.graphs.clear()
+        self.graph_vars = None
+        torch.cuda.synchronize()
+
+    def call(self, method_name, *args):
+        return getattr(self, method_name)(*args)
+
+    # ------------------------------------------------------------------ set-up
+    def warmup_model(self):
+        """One worst-case prefill before the cache exists, to learn the activation peak
+        (model_runner.py:108-116); it also allocates the kernels' workspaces."""
+        torch.cuda.empty_cache()
+        torch.cuda.reset_peak_memory_stats()
+        cfg = self.config
+        num_seqs = max(1, min(cfg.max_num_batched_tokens // cfg.max_model_len, cfg.max_num_seqs))
+        seqs = [Sequence([0] * cfg.max_model_len) for _ in range(num_seqs)]
+        self.run(seqs, True)
+        torch.cuda.empty_cache()
+
+    def kv_block_bytes(self) -> int:
+        hf = self.config.hf_config
+        itemsize = 2 if self.kv_dtype == torch.bfloat16 else 1
+        return 2 * hf.num_hidden_layers * self.block_size * hf.num_key_value_heads * hf.head_dim * itemsize
+
+    def allocate_kv_cache(self):
+        """One tensor ``[2, L, nblk, block, Hkv, Dh]``; layer l gets views ``kv[0, l]`` / ``kv[1, l]``
+        (model_runner.py:118-139).  ``num_kvcache_blocks`` may be fixed in the config."""
+        cfg, hf = self.config, self.config.hf_config
+        if cfg.num_kvcache_blocks <= 0:
+            free, total = torch.cuda.mem_get_info()
+            used = total - free
+            stats = torch.cuda.memory_stats()
+            peak, current = stats["allocated_bytes.all.peak"], stats["allocated_bytes.all.current"]
+            cfg.num_kvcache_blocks = int(total * cfg.gpu_memory_utilization - used - (peak - current)) // self.kv_block_bytes()
+        assert cfg.num_kvcache_blocks > 0
+        self.kv_cache = torch.zeros(2, hf.num_hidden_layers, cfg.num_kvcache_blocks, self.block_size,
+                                    hf.num_key_value_heads, hf.head_dim, dtype=self.kv_dtype, device=self.device)
+        layer_id = 0
+        for module in self.model.modules():
+            if hasattr(module, "k_cache") and hasattr(module, "v_cache"):
+                module.k_cache = self.kv_cache[0, layer_id]
+                module.v_cache = self.kv_cache[1, layer_id]
+                if self.kv_dtype != torch.bfloat16:
+                    # build-defined static per-head scales for the e4m3 cache
+                    module.k_scale = torch.full((hf.num_key_value_heads,), 1.0 / 16, dtype=torch.float32, device=self.device)
+                    module.v_scale = torch.full((hf.num_key_value_heads,), 1.0 / 16, dtype=torch.float32, device=self.device)
+                layer_id += 1
+
+    # ------------------------------------------------------------------ per-step inputs
+    def _upload(self, arrays: dict) -> dict:
+        """All integer inputs of a step go through ONE pinned staging buffer and ONE H2D copy."""
+        names = [k for k, v in arrays.items() if isinstance(v, np.ndarray)]
+        offs, total = {}, 0
+        for k in names:
+            total = (total + 15) // 16 * 16
+            offs[k] = total
+            total += arrays[k].nbytes
+        stage = torch.empty(max(total, 16), dtype=torch.uint8, pin_memory=True)
+        sv = stage.numpy()
+        for k in names:
+            sv[offs[k]:offs[k] + arrays[k].nbytes] = arrays[k].reshape(-1).view(np.uint8)
+        dev = stage.to(self.device, non_blocking=True)
+        out = dict(arrays)
+        for k in names:
+            a = arrays[k]
+            dt = {np.dtype("int64"): torch.int64, np.dtype("int32"): torch.int32, np.dtype("float32"): torch.float32}[a.dtype]
+            out[k] = dev[offs[k]:offs[k] + a.nbytes].view(dt).view(*a.shape)
+        return out
+
+    def prepare_block_tables(self, seqs):
+        return torch.from_numpy(I.block_tables_array(seqs)).to(self.device)
+
+    def prepare_prefill(self, seqs):
+        d = self._upload(I.prefill_inputs(seqs, self.block_size))
+        set_context(True, d["cu_seqlens_q"], d["cu_seqlens_k"], d["max_seqlen_q"], d["max_seqlen_k"],
+                    d["slot_mapping"], None, d["block_tables"])
+        return d["input_ids"], d["positions"]
+
+    def prepare_decode(self, seqs):
+        d = self._upload(I.decode_inputs(seqs, self.block_size, self.config.decode_position_quirk))
+        set_context(False, slot_mapping=d["slot_mapping"], context_lens=d["context_lens"], block_tables=d["block_tables"])
+        return d["input_ids"], d["positions"]
+
+    def prepare_sample(self, seqs):
+        t = np.asarray([s.temperature for s in seqs], dtype=np.float32)
+        self._all_greedy = bool((t == 0).all())
+        return torch.from_numpy(t).to(self.device, non_blocking=True)
+
+    # ------------------------------------------------------------------ forward
+    @torch.inference_mode()
+    def run_model(self, input_ids, positions, is_prefill):
+        bs = input_ids.size(0)
+        if is_prefill or self.enforce_eager or not self.graph_bs or bs > self.graph_bs[-1]:
+            return self.model.compute_logits(self.model(input_ids, positions))
+        ctx = get_context()
+        gbs = next(x for x in self.graph_bs if x >= bs)
+        gv = self.graph_vars
+        if gbs != bs:      # padding rows: slot -1 (no cache write), length 0 (no cache read)
+            gv["slot_mapping"][bs:gbs].fill_(-1)
+            gv["context_lens"][bs:gbs].zero_()
+            gv["input_ids"][bs:gbs].zero_()
+            gv["positions"][bs:gbs].zero_()
+        gv["input_ids"][:bs] = input_ids
+        gv["positions"][:bs] = positions
+        gv["slot_mapping"][:bs] = ctx.slot_mapping
+        gv["context_lens"][:bs] = ctx.context_lens
+        w = ctx.block_tables.size(1)
+        gv["block_tables"][:bs, :w] = ctx.block_tables
+        self.graphs[gbs].replay()
+        return self.model.compute_logits(gv["outputs"][:bs])
+
+    def run(self, seqs, is_prefill):
+        input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
+        temperatures = self.prepare_sample(seqs)
+        logits = self.run_model(input_ids, positions, is_prefill)
+        token_ids = self.sampler(logits, temperatures, self._all_greedy).tolist()   # the step's one device sync
+        reset_context()
+        return token_ids
+
+    # ------------------------------------------------------------------ hipGraph capture
+    @torch.inference_mode()
+    def capture_graphs(self):
+        """Capture ``model(input_ids, positions)`` for batch buckets 1, 2, 4, 8, 16, 32, ... (model_runner.py:272-308).
+        Every kernel of the hot path takes its geometry from the static shapes only, so a replay
+        is valid for any lengths and block tables written into the static buffers."""
+        cfg, hf = self.config, self.config.hf_config
+        max_bs = min(cfg.max_num_seqs, 512)
+        max_blocks = (cfg.max_model_len + self.block_size - 1) // self.block_size
+        dev = self.device
+        gv = dict(
+            input_ids=torch.zeros(max_bs, dtype=torch.int64, device=dev),
+            positions=torch.zeros(max_bs, dtype=torch.int64, device=dev),
+            slot_mapping=torch.full((max_bs,), -1, dtype=torch.int32, device=dev),
+            context_lens=torch.zeros(max_bs, dtype=torch.int32, device=dev),
+            block_tables=torch.zeros(max_bs, max_blocks, dtype=torch.int32, device=dev),
+            outputs=torch.zeros(max_bs, hf.hidden_size, dtype=hf.torch_dtype, device=dev),
+        )
+        self.graph_bs = [b for b in (1, 2, 4, 8) if b <= max_bs] + list(range(16, max_bs + 1, 16))
+        pool = None
+        for bs in reversed(self.graph_bs):
+            graph = torch.cuda.CUDAGraph()
+            set_context(False, slot_mapping=gv["slot_mapping"][:bs], context_lens=gv["context_lens"][:bs],
+                        block_tables=gv["block_tables"][:bs, :])
+            gv["outputs"][:bs] = self.model(gv["input_ids"][:bs], gv["positions"][:bs])    # warm-up
+            with torch.cuda.graph(graph, pool):
+                gv["outputs"][:bs] = self.model(gv["input_ids"][:bs], gv["positions"][:bs])
+            if pool is None:
+                pool = graph.pool()
+            self.graphs[bs] = graph
+            torch.cuda.synchronize()
+            reset_context()
+        self.graph_vars = gv

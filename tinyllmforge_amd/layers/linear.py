@@ -1,0 +1,126 @@
+"""Linear layers (reference: tinyvllm/layers/linear.py:10-184).
+
+Same class names, weight layout (``[out, in]``, ``nn.Linear`` order) and ``weight_loader``
+protocol as the reference; this build runs one GPU, so the tensor-parallel rank is 0 of 1 and
+there is no all-reduce.  ``quantize_()`` swaps the bf16 weight for an int8 weight plus a
+per-output-channel fp32 scale; ``forward`` then runs the weight-only int8 GEMM.
+"""
+import torch
+from torch import nn
+
+from .. import ops
+
+
+def quantize_per_channel(weight: torch.Tensor):
+    """Symmetric int8: ``scale[n] = max|W[n,:]| / 127``, ``Wq = clamp(round(W / scale), -127, 127)``."""
+    w = weight.float()
+    amax = w.abs().amax(dim=1)
+    scale = torch.where(amax > 0, amax / 127.0, torch.ones_like(amax))
+    wq = torch.round(w / scale[:, None]).clamp_(-127, 127).to(torch.int8)
+    return wq.contiguous(), scale.contiguous()
+
+
+class LinearBase(nn.Module):
+    def __init__(self, input_size: int, output_size: int, tp_dim: int | None = None):
+        super().__init__()
+        self.input_size = input_size
+        self.output_size = output_size
+        self.tp_dim = tp_dim
+        self.tp_rank = 0
+        self.tp_size = 1
+        self.qweight = None
+        self.qscale = None
+
+    def _make_params(self, out_features: int, in_features: int, bias: bool):
+        self.weight = nn.Parameter(torch.empty(out_features, in_features))
+        self.weight.weight_loader = self.weight_loader
+        if bias:
+            self.bias = nn.Parameter(torch.empty(out_features))
+            self.bias.weight_loader = self.weight_loader
+        else:
+            self.register_parameter("bias", None)
+
+    def quantize_(self):
+        """Replace the bf16 weight by int8 + scale (frees the bf16 copy)."""
+        self.qweight, self.qscale = quantize_per_channel(self.weight.data)
+        self.weight.data = torch.empty(0, dtype=self.weight.dtype, device=self.weight.device)
+        return self
+
+    def load_quantized(self, qweight: torch.Tensor, qscale: torch.Tensor):
+        self.qweight, self.qscale = qweight.contiguous(), qscale.contiguous()
+        self.weight.data = torch.empty(0, dtype=self.weight.dtype, device=qweight.device)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.qweight is not None:
+            y = ops.w8a16_linear(x, self.qweight, self.qscale)
+        else:
+            y = ops.bf16_linear(x, self.weight.data)
+        if self.bias is not None:
+            y = y + self.bias
+        return y
+
+
+class ReplicatedLinear(LinearBase):
+    def __init__(self, input_size: int, output_size: int, bias: bool = False):
+        super().__init__(input_size, output_size)
+        self._make_params(output_size, input_size, bias)
+
+    def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor):
+        param.data.copy_(loaded_weight)
+
+
+class ColumnParallelLinear(LinearBase):
+    def __init__(self, input_size: int, output_size: int, bias: bool = False):
+        super().__init__(input_size, output_size, 0)
+        self.input_size_per_partition = input_size
+        self.output_size_per_partition = output_size // self.tp_size
+        self._make_params(self.output_size_per_partition, input_size, bias)
+
+    def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor):
+        n = param.data.size(self.tp_dim)
+        param.data.copy_(loaded_weight.narrow(self.tp_dim, self.tp_rank * n, n))
+
+
+class MergedColumnParallelLinear(ColumnParallelLinear):
+    """Several projections stacked along the output dim (gate_up_proj)."""
+
+    def __init__(self, input_size: int, output_sizes: list[int], bias: bool = False):
+        self.output_sizes = output_sizes
+        super().__init__(input_size, sum(output_sizes), bias=bias)
+
+    def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor, loaded_shard_id: int):
+        offset = sum(self.output_sizes[:loaded_shard_id]) // self.tp_size
+        size = self.output_sizes[loaded_shard_id] // self.tp_size
+        dst = param.data.narrow(self.tp_dim, offset, size)
+        dst.copy_(loaded_weight.chunk(self.tp_size, self.tp_dim)[self.tp_rank])
+
+
+class QKVParallelLinear(ColumnParallelLinear):
+    """q, k and v projections stacked as [q | k | v] along the output dim."""
+
+    def __init__(self, hidden_size: int, head_size: int, total_num_heads: int,
+                 total_num_kv_heads: int | None = None, bias: bool = False):
+        self.head_size = head_size
+        self.total_num_heads = total_num_heads
+        self.total_num_kv_heads = total_num_kv_heads or total_num_heads
+        self.num_heads = self.total_num_heads
+        self.num_kv_heads = self.total_num_kv_heads
+        super().__init__(hidden_size, (self.num_heads + 2 * self.num_kv_heads) * head_size, bias)
+
+    def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor, loaded_shard_id: str):
+        assert loaded_shard_id in ("q", "k", "v")
+        q_size, kv_size = self.num_heads * self.head_size, self.num_kv_heads * self.head_size
+        offset, size = {"q": (0, q_size), "k": (q_size, kv_size), "v": (q_size + kv_size, kv_size)}[loaded_shard_id]
+        dst = param.data.narrow(self.tp_dim, offset, size)
+        dst.copy_(loaded_weight.chunk(self.tp_size, self.tp_dim)[self.tp_rank])
+
+
+class RowParallelLinear(LinearBase):
+    def __init__(self, input_size: int, output_size: int, bias: bool = False):
+        super().__init__(input_size, output_size, 1)
+        self.input_size_per_partition = input_size // self.tp_size
+        self._make_params(output_size, self.input_size_per_partition, bias)
+
+    def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor):
+        n = param.data.size(self.tp_dim)
+        param.data.copy_(loaded_weight.narrow(self.tp_dim, self.tp_rank * n, n))
