@@ -102,6 +102,32 @@ def time_launches(fn, steps, warmup):
                 span_ms=span, wall_s=wall)
 
 
+def time_graph(fn, launches=20, replays=20):
+    """Mean GPU time (ms) of one call of ``fn`` when ``launches`` calls are captured into a hipGraph and
+    replayed: short kernels are timed back to back, without the host's per-call launch cost."""
+    import torch
+    fn()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        fn()
+        with torch.cuda.graph(g, stream=s):
+            for _ in range(launches):
+                fn()
+    torch.cuda.synchronize()
+    g.replay()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(replays):
+        g.replay()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / (launches * replays)
+
+
 def bench_probes(args):
     """Rate of a plain read-only and a plain copy kernel over 1 GiB: the practical HBM ceiling of the box."""
     import torch
@@ -182,8 +208,7 @@ def bench_gemm(args, ms=(1, 16, 64, 256, 2048)):
         scale = torch.rand(N, device="cuda") * 9e-3 + 1e-3
         for M in ms:
             x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
-            t = time_launches(lambda: P.w8a16_linear(x, wq, scale), max(20, args.steps // 4), 10)
-            sec = t["mean_ms"] * 1e-3
+            sec = time_graph(lambda: P.w8a16_linear(x, wq, scale)) * 1e-3
             nbytes = N * K + 4 * N + 2 * M * K + 2 * M * N
             flops = 2.0 * M * N * K
             bound = "hbm" if M <= 64 else "mfma"

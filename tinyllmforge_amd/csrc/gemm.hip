@@ -20,12 +20,16 @@
 // (each with a private L2), so workgroup b belongs to XCD b % 8.  Each XCD is
 // given whole columns of N-tiles and walks the M-tiles of a column first, so
 // the workgroups that share an L2 share W panels and step through K together.
+#include <stdio.h>
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace tlf {
 
 constexpr int kBK = 64;           // K elements per LDS tile
 constexpr int kLdsK = kBK + 8;    // padded LDS row: 144 B
+constexpr int kSkinnyMaxM = 16;   // at or below this many tokens the skinny kernel runs
 
 template <int ROWS, bool W8>
 struct TileLoader;
@@ -237,44 +241,239 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmParams p) 
   *reinterpret_cast<uint2 *>(p.y + i4 * 4) = st;
 }
 
+// ---------------------------------------------------------------------------
+// Skinny GEMM for a handful of tokens (decode at small batch; up to 64 rows): weight-bandwidth bound.
+//
+// W is streamed exactly once, straight from HBM into MFMA A-operand registers
+// (non-temporal 128-bit loads, no LDS staging): lane (r, g) of a wave loads 16
+// consecutive K elements of channel r; the K index inside an MFMA is only a
+// summation label, so the two halves of that load feed two
+// v_mfma_f32_16x16x32_bf16 whose B operand (the activations, read from L2) uses
+// the same labelling.  A workgroup owns 16*TN output channels; its 8 waves split
+// K and the partial accumulators are summed through LDS, so nothing but the
+// final bf16 rows goes back to memory.
+template <int MT, int TN, bool W8>
+__global__ __launch_bounds__(512) void skinny_gemm_kernel(const GemmParams p) {
+  constexpr int kWaves = 8;
+  constexpr int kU = 4;  // K-blocks of 64 whose weight loads are in flight together
+  __shared__ __attribute__((aligned(16))) float red[kWaves][TN * MT][64][4];
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16 * TN;
+  const int nkb = p.K / kBK;
+  const int kb_begin = static_cast<int>(static_cast<int64_t>(nkb) * wave / kWaves);
+  const int kb_end = static_cast<int>(static_cast<int64_t>(nkb) * (wave + 1) / kWaves);
+  const int64_t ldw = W8 ? p.K : static_cast<int64_t>(p.K) * 2;  // bytes per weight row
+
+  floatx4 acc[TN][MT];
+#pragma unroll
+  for (int t = 0; t < TN; ++t)
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[t][m] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const unsigned char *wrow[TN];
+  bool wok[TN];
+#pragma unroll
+  for (int t = 0; t < TN; ++t) {
+    const int n = n0 + t * 16 + r;
+    wok[t] = n < p.N;
+    wrow[t] = p.w + static_cast<int64_t>(wok[t] ? n : 0) * ldw;
+  }
+  const unsigned char *xrow[MT];
+  bool xok[MT];
+#pragma unroll
+  for (int m = 0; m < MT; ++m) {
+    const int row = m * 16 + r;
+    xok[m] = row < p.M;
+    xrow[m] = p.x + static_cast<int64_t>(xok[m] ? row : 0) * p.ldx_bytes;
+  }
+
+  for (int kb0 = kb_begin; kb0 < kb_end; kb0 += kU) {
+    // issue the weight loads of up to kU K-blocks
+    uint4 wraw[kU][TN][W8 ? 1 : 2];
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      const int kb = kb0 + u;
+#pragma unroll
+      for (int t = 0; t < TN; ++t) {
+        if (W8) {
+          wraw[u][t][0] = make_uint4(0, 0, 0, 0);
+          if (kb < kb_end && wok[t]) wraw[u][t][0] = load_nt_u4(wrow[t] + kb * kBK + g * 16);
+        } else {
+          wraw[u][t][0] = make_uint4(0, 0, 0, 0);
+          wraw[u][t][W8 ? 0 : 1] = make_uint4(0, 0, 0, 0);
+          if (kb < kb_end && wok[t]) {
+            const unsigned char *src = wrow[t] + (static_cast<int64_t>(kb) * kBK + g * 16) * 2;
+            wraw[u][t][0] = load_nt_u4(src);
+            wraw[u][t][W8 ? 0 : 1] = load_nt_u4(src + 16);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kU; ++u) {
+      const int kb = kb0 + u;
+      if (kb >= kb_end) break;  // uniform per wave
+      bf16x8 a0[TN], a1[TN];
+#pragma unroll
+      for (int t = 0; t < TN; ++t) {
+        Pack16 lo, hi;
+        if (W8) {
+          const uint4 q = wraw[u][t][0];
+          const uint2 c0 = TileLoader<64, true>::cvt4(q.x), c1 = TileLoader<64, true>::cvt4(q.y);
+          const uint2 c2 = TileLoader<64, true>::cvt4(q.z), c3 = TileLoader<64, true>::cvt4(q.w);
+          lo.u = make_uint4(c0.x, c0.y, c1.x, c1.y);
+          hi.u = make_uint4(c2.x, c2.y, c3.x, c3.y);
+        } else {
+          lo.u = wraw[u][t][0];
+          hi.u = wraw[u][t][W8 ? 0 : 1];
+        }
+        a0[t] = lo.v;
+        a1[t] = hi.v;
+      }
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        Pack16 b0, b1;
+        b0.u = make_uint4(0, 0, 0, 0);
+        b1.u = make_uint4(0, 0, 0, 0);
+        if (xok[m]) {
+          const unsigned char *src = xrow[m] + (static_cast<int64_t>(kb) * kBK + g * 16) * 2;
+          b0.u = *reinterpret_cast<const uint4 *>(src);
+          b1.u = *reinterpret_cast<const uint4 *>(src + 16);
+        }
+#pragma unroll
+        for (int t = 0; t < TN; ++t) {
+          acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[t], b0.v, acc[t][m], 0, 0, 0);
+          acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[t], b1.v, acc[t][m], 0, 0, 0);
+        }
+      }
+    }
+  }
+  // acc[t][m]: token m*16 + r, channels n0 + t*16 + 4g + i
+#pragma unroll
+  for (int t = 0; t < TN; ++t)
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+      *reinterpret_cast<float4 *>(&red[wave][t * MT + m][lane][0]) =
+          make_float4(acc[t][m][0], acc[t][m][1], acc[t][m][2], acc[t][m][3]);
+  __syncthreads();
+  for (int item = tid; item < TN * MT * 64; item += 512) {
+    const int tile = item >> 6, l = item & 63;
+    const int t = tile / MT, m = tile % MT;
+    float4 s = *reinterpret_cast<const float4 *>(&red[0][tile][l][0]);
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) {
+      const float4 v = *reinterpret_cast<const float4 *>(&red[w][tile][l][0]);
+      s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+    }
+    const int token = m * 16 + (l & 15);
+    const int n = n0 + t * 16 + (l >> 4) * 4;
+    if (token >= p.M || n >= p.N) continue;
+    if (W8) {
+      const float4 sc = *reinterpret_cast<const float4 *>(p.scale + n);
+      s.x *= sc.x; s.y *= sc.y; s.z *= sc.z; s.w *= sc.w;
+    }
+    uint2 st;
+    st.x = pack_bf16x2(s.x, s.y);
+    st.y = pack_bf16x2(s.z, s.w);
+    *reinterpret_cast<uint2 *>(p.y + static_cast<int64_t>(token) * p.N + n) = st;
+  }
+}
+
+template <bool W8>
+int launch_skinny(const GemmParams &p, hipStream_t stream) {
+  const int mt = (p.M + 15) / 16;
+  const int tiles16 = (p.N + 15) / 16;
+  // more channels per workgroup reuse the activation fragments, as long as the grid stays large
+  int tn = 1;
+  if (tiles16 >= 4 * 512) tn = 4;
+  else if (tiles16 >= 2 * 512) tn = 2;
+  const dim3 grid((tiles16 + tn - 1) / tn);
+#define TLF_SK(MT_, TN_) \
+  hipLaunchKernelGGL((skinny_gemm_kernel<MT_, TN_, W8>), grid, dim3(512), 0, stream, p)
+#define TLF_SK_TN(MT_)          \
+  if (tn == 4) TLF_SK(MT_, 4);  \
+  else if (tn == 2) TLF_SK(MT_, 2); \
+  else TLF_SK(MT_, 1)
+  switch (mt) {
+    case 1: TLF_SK_TN(1); break;
+    case 2: TLF_SK_TN(2); break;
+    case 3: TLF_SK_TN(3); break;
+    default: TLF_SK_TN(4); break;
+  }
+#undef TLF_SK_TN
+#undef TLF_SK
+  return launch_status();
+}
+
 struct GemmPlan {
   int bn, bm;   // tile
   int splits;   // split-K factor
   int k_per_split;
 };
 
-// Fill the 256 CUs: largest tile whose grid still has >= ~1 workgroup per CU,
-// then split K when even the smallest tile leaves CUs idle.
+// Tile and split-K choice, from a sweep over the Qwen3-8B projection shapes on MI355X.
+// A K-tile step of this kernel costs roughly the same whatever the tile (it is latency bound),
+// so mid-size problems want many small tiles plus a moderate split of K (each split keeps at
+// least 16 K-tiles), and only problems with thousands of tiles use the large MFMA-friendly tiles.
 inline GemmPlan plan_gemm(int M, int N, int K) {
   GemmPlan g;
-  const int cus = 256;
   auto tiles = [&](int bn, int bm) { return ((N + bn - 1) / bn) * ((M + bm - 1) / bm); };
-  if (M > 128 && tiles(256, 256) >= cus) {
-    g.bn = 256; g.bm = 256;
-  } else if (M > 64 && tiles(128, 128) >= cus) {
-    g.bn = 128; g.bm = 128;
-  } else if (M > 64) {
-    g.bn = 128; g.bm = 128;
-  } else {
-    g.bn = 128; g.bm = 64;
-  }
-  const int t = tiles(g.bn, g.bm);
-  int splits = 1;
+  auto pow2_floor = [](int v) { int p = 1; while (p * 2 <= v) p *= 2; return p; };
   const int ktiles = K / kBK;
-  while (t * splits * 2 <= cus * 2 && splits * 2 <= 16 && ktiles / (splits * 2) >= 4) splits *= 2;
-  if (t >= cus) splits = 1;
-  g.splits = splits;
+  const int max_split = ktiles / 16 > 1 ? pow2_floor(ktiles / 16) : 1;
+  int splits = 1;
+  if (tiles(64, 64) <= 512) {
+    g.bn = 64; g.bm = 64;
+    splits = pow2_floor(1024 / tiles(64, 64));
+  } else if (tiles(128, 128) <= 1024) {
+    g.bn = 128; g.bm = 128;
+    splits = tiles(128, 128) <= 256 ? pow2_floor(512 / tiles(128, 128)) : 1;
+  } else if (tiles(256, 256) >= 256) {
+    g.bn = 256; g.bm = 256;
+  } else {
+    g.bn = 128; g.bm = 128;
+  }
+  if (splits > max_split) splits = max_split;
+  if (splits > 16) splits = 16;
+  if (splits < 1) splits = 1;
   const int kt_per = (ktiles + splits - 1) / splits;
   g.k_per_split = kt_per * kBK;
   g.splits = (ktiles + kt_per - 1) / kt_per;
   return g;
 }
 
+// TLF_GEMM_PLAN="bn,bm,splits" forces one plan (tuning sweeps); TLF_GEMM_SKINNY_MAX_M moves the
+// hand-over point between the skinny and the tiled kernel.
+inline bool plan_override(GemmPlan &g, int K) {
+  const char *e = getenv("TLF_GEMM_PLAN");
+  if (!e) return false;
+  int bn = 0, bm = 0, sp = 0;
+  if (sscanf(e, "%d,%d,%d", &bn, &bm, &sp) != 3) return false;
+  const int ktiles = K / kBK;
+  if (sp < 1) sp = 1;
+  if (sp > ktiles) sp = ktiles;
+  const int kt_per = (ktiles + sp - 1) / sp;
+  g.bn = bn; g.bm = bm;
+  g.k_per_split = kt_per * kBK;
+  g.splits = (ktiles + kt_per - 1) / kt_per;
+  return true;
+}
+
+inline int skinny_max_m() {
+  static int v = -1;
+  if (v < 0) {
+    v = kSkinnyMaxM;
+    if (const char *e = getenv("TLF_GEMM_SKINNY_MAX_M")) v = atoi(e);
+  }
+  return v;
+}
+
 template <bool W8>
 int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *scale, void *y,
                 int32_t M, int32_t N, int32_t K, void *workspace, size_t workspace_bytes,
                 hipStream_t stream) {
-  const GemmPlan g = plan_gemm(M, N, K);
   GemmParams p;
   p.x = static_cast<const unsigned char *>(x);
   p.ldx_bytes = x_stride * 2;
@@ -283,6 +482,12 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   p.y = static_cast<unsigned short *>(y);
   p.partial = nullptr;
   p.M = M; p.N = N; p.K = K;
+  if (M <= skinny_max_m()) {
+    p.k_per_split = K; p.splits = 1; p.m_tiles = 1; p.n_tiles = 1;
+    return launch_skinny<W8>(p, stream);
+  }
+  GemmPlan g = plan_gemm(M, N, K);
+  plan_override(g, K);
   p.k_per_split = g.k_per_split;
   p.splits = g.splits;
   p.m_tiles = (M + g.bm - 1) / g.bm;
@@ -294,12 +499,22 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
     p.partial = static_cast<float *>(workspace);
   }
   const dim3 grid(((p.n_tiles + 7) / 8) * 8 * p.m_tiles, g.splits);
-  if (g.bn == 256 && g.bm == 256)
-    hipLaunchKernelGGL((gemm_kernel<256, 256, 2, 2, W8>), grid, dim3(256), 0, stream, p);
-  else if (g.bn == 128 && g.bm == 128)
-    hipLaunchKernelGGL((gemm_kernel<128, 128, 2, 2, W8>), grid, dim3(256), 0, stream, p);
-  else
-    hipLaunchKernelGGL((gemm_kernel<128, 64, 4, 1, W8>), grid, dim3(256), 0, stream, p);
+#define TLF_TILE(BN_, BM_, WN_, WM_)                                                          \
+  if (g.bn == BN_ && g.bm == BM_) {                                                           \
+    hipLaunchKernelGGL((gemm_kernel<BN_, BM_, WN_, WM_, W8>), grid, dim3(256), 0, stream, p); \
+    launched = true;                                                                          \
+  }
+  bool launched = false;
+  TLF_TILE(256, 256, 2, 2)
+  TLF_TILE(128, 256, 2, 2)
+  TLF_TILE(64, 256, 1, 4)
+  TLF_TILE(256, 128, 2, 2)
+  TLF_TILE(128, 128, 2, 2)
+  TLF_TILE(64, 128, 1, 4)
+  TLF_TILE(128, 64, 4, 1)
+  TLF_TILE(64, 64, 2, 2)
+#undef TLF_TILE
+  if (!launched) return TLF_E_UNSUPPORTED;
   int rc = launch_status();
   if (rc != TLF_OK) return rc;
   if (g.splits > 1) {
@@ -325,9 +540,9 @@ using namespace tlf;
 
 extern "C" size_t tlf_w8a16_gemm_workspace_bytes(int32_t M, int32_t N, int32_t K) {
   if (M <= 0 || N <= 0 || K <= 0 || K % kBK) return 0;
-  const GemmPlan g = plan_gemm(M, N, K);
-  if (g.splits <= 1) return 0;
-  return static_cast<size_t>(g.splits) * M * N * sizeof(float);
+  // room for the deepest split any plan may use (16), so that tuning overrides stay in bounds
+  if (M <= skinny_max_m()) return 0;
+  return static_cast<size_t>(16) * M * N * sizeof(float);
 }
 
 extern "C" int tlf_w8a16_gemm(const void *x, int64_t x_stride, const void *wq, const float *scale,

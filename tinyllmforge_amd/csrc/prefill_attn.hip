@@ -117,7 +117,7 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p
   constexpr int kChunks = KV8 ? 8 : 16;
   constexpr int kPasses = kBKV * kChunks / 256;
   uint4 kreg[kPasses], vreg[kPasses];
-  auto load_tile = [&](int kv0) {
+  auto load_tile = [&](int kv0) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < kPasses; ++i) {
       const int t = i * (256 / kChunks) + tid / kChunks;
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p
       }
     }
   };
-  auto store_tile = [&]() {
+  auto store_tile = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < kPasses; ++i) {
       const int t = i * (256 / kChunks) + tid / kChunks;
@@ -175,7 +175,7 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p
 
   load_tile(0);
   store_tile();
-  __syncthreads();
+  lds_barrier();
   for (int kv0 = 0; kv0 < kv_end; kv0 += kBKV) {
     const bool more = kv0 + kBKV < kv_end;
     if (more) load_tile(kv0 + kBKV);
@@ -255,10 +255,10 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p
         }
       }
     }
-    __syncthreads();
+    lds_barrier();
     if (more) {
       store_tile();
-      __syncthreads();
+      lds_barrier();
     }
   }
 
