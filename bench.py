@@ -1,21 +1,30 @@
 #!/usr/bin/env python3
 """Benchmark of the per-token hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode_attn|gemm|all]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload e2e|decode_attn|gemm|all]
 
-Prints ONE JSON line.  A "step" is one pass of the hot-path kernel over one batch of
-synthetic input that is already resident in HBM.  The default workload is the paged
-decode attention microbench of BASELINE.json configs[1]:
+Prints ONE JSON line.
 
-    B=64, Hq=32, Hkv=8, Dh=128, block_size=256, ctx ~ U[512, 4096], seed 0,
-    2048-block pool, block tables = prefix of randperm(2048), K/V rows N(0,1) bf16
-    written through the KV-store kernel, softmax scale 1/sqrt(128).
+``value`` (default workload ``e2e``) is BASELINE.json's headline metric: output tokens/s of a
+Qwen3-8B-shaped decoder (36 layers, hidden 4096, 32 query / 8 KV heads, head_dim 128,
+intermediate 12288, vocab 151936; random-init weights, W8A16 linears; the bf16 run is reported
+beside it) on the reference's own bench.py recipe (tinyvllm bench.py:39-59): ``seed(0)``, 256
+prompts of ``randint(100, 1024)`` random token ids, ``max_tokens = randint(100, 1024)``,
+``ignore_eos``, continuous batching, hipGraph-captured decode, one warm-up ``generate`` first;
+tok/s = sum(max_tokens) / wall time of ``generate()``, prefill included.  Greedy sampling
+(temperature 0; the reference's script uses 0.6) keeps the run deterministic.  A "step" is one
+engine step (one prefill or one decode pass over the running batch); ``--steps K`` stops the
+timed run after K engine steps (0 = the whole job).
 
-``roofline`` is measured live with HIP events on the launch stream: algorithmic bytes per
-launch (sum_b ctx_b * Hkv*Dh*2(K,V)*2 B + q and out + tables) over the mean launch time,
-against the 8 TB/s HBM peak.  ``cpu_baseline`` times the CPU oracle (this repo's
-restatement of the reference op; the checker, never the product) on a bounded sample of
-the same workload on the host cores of the box.
+``roofline`` is the paged decode attention kernel, the largest single consumer of a decode step,
+measured live with HIP events on its launch stream on BASELINE.json configs[1]
+(B=64, Hq=32, Hkv=8, Dh=128, block 256, ctx ~ U[512, 4096], 2048-block pool, seed 0):
+algorithmic bytes per launch (sum_b ctx_b * Hkv*Dh*2(K,V)*2 B + q and out + tables) over the
+mean launch time, against the 8 TB/s HBM peak.
+
+``cpu_baseline`` times the CPU oracle (this repo's restatement of the reference's PyTorch layer
+semantics; the checker, never the product) on a bounded sample of the same workload on the box's
+host cores.
 """
 from __future__ import annotations
 
@@ -36,9 +45,11 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=30)
-    ap.add_argument("--workload", default="decode_attn", choices=["decode_attn", "gemm", "all"])
+    ap.add_argument("--steps", type=int, default=0, help="timed engine steps of the e2e run (0 = whole job)")
+    ap.add_argument("--warmup", type=int, default=1, help="warm-up generate() calls before the timed run")
+    ap.add_argument("--workload", default="e2e", choices=["e2e", "decode_attn", "gemm", "all"])
+    ap.add_argument("--attn-steps", type=int, default=200, help="timed launches of the decode-attention microbench")
+    ap.add_argument("--num-seqs", type=int, default=256)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--batch", type=int, default=64)
     return ap.parse_args()
@@ -153,9 +164,9 @@ def bench_decode_attn(args):
         return P.paged_decode_attention(case["q"], case["k_cache"], case["v_cache"], case["ctx"], case["bt"],
                                         case["scale"])
 
-    t = time_launches(step, args.steps, args.warmup)
+    t = time_launches(step, args.attn_steps, 30)
     # "step" time = back-to-back launches over the timed region (what a decode loop sees)
-    ms_per_step = t["span_ms"] / args.steps
+    ms_per_step = t["span_ms"] / args.attn_steps
     gbps = case["algo_bytes"] / (ms_per_step * 1e-3) / 1e9
     kern_gbps = case["algo_bytes"] / (t["mean_ms"] * 1e-3) / 1e9
     res = dict(ms_per_step=ms_per_step, value=gbps,
@@ -219,6 +230,88 @@ def bench_gemm(args, ms=(1, 16, 64, 256, 2048)):
     return rows
 
 
+# ----------------------------------------------------------------------------- config 4 (end to end)
+def e2e_workload(num_seqs=256):
+    """The reference's bench.py recipe (pure-python ``random``: platform independent)."""
+    from random import randint, seed
+    seed(0)
+    prompts = [[randint(0, 10000) for _ in range(randint(100, 1024))] for _ in range(num_seqs)]
+    max_tokens = [randint(100, 1024) for _ in range(num_seqs)]
+    return prompts, max_tokens
+
+
+def bench_e2e(args, quantization):
+    import torch
+    from tinyllmforge_amd import LLM, SamplingParams
+    prompts, max_tokens = e2e_workload(args.num_seqs)
+    t0 = time.perf_counter()
+    llm = LLM("qwen3-8b", enforce_eager=False, max_model_len=4096, quantization=quantization,
+              gpu_memory_utilization=0.6, seed=0)
+    init_s = time.perf_counter() - t0
+    sps = [SamplingParams(temperature=0.0, ignore_eos=True, max_tokens=m) for m in max_tokens]
+    for _ in range(max(1, args.warmup)):
+        llm.generate([[1, 2, 3, 4, 5, 6, 7, 8]], SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    if args.steps > 0:                       # a bounded number of engine steps
+        for p, sp in zip(prompts, sps):
+            llm.add_request(p, sp)
+        produced, steps = 0, 0
+        while not llm.is_finished() and steps < args.steps:
+            seqs, is_prefill = llm.scheduler.schedule()
+            toks = llm.model_runner.call("run", seqs, is_prefill)
+            llm.scheduler.postprocess(seqs, toks)
+            produced += len(seqs)          # every scheduled sequence gains one token, prefill or decode
+            steps += 1
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        total, stats = produced, dict(steps=steps)
+        # drain what is left so that the engine can be torn down cleanly
+        while not llm.is_finished():
+            llm.step()
+    else:
+        llm.generate(prompts, sps)
+        torch.cuda.synchronize()
+        wall = time.perf_counter() - t0
+        total = sum(max_tokens)
+        st = llm.last_stats
+        stats = dict(steps=st["prefill_steps"] + st["decode_steps"], prefill_steps=st["prefill_steps"],
+                     decode_steps=st["decode_steps"], prefill_s=round(st["prefill_time"], 3),
+                     decode_s=round(st["decode_time"], 3),
+                     decode_ms_per_step=round(1e3 * st["decode_time"] / max(1, st["decode_steps"]), 3))
+    model_params = {k: v.data for k, v in llm.model_runner.model.named_parameters()} if quantization is None else None
+    res = dict(tok_s=total / wall, wall_s=wall, total_output_tokens=total, init_s=round(init_s, 1), stats=stats,
+               kv_blocks=llm.config.num_kvcache_blocks)
+    cpu = None
+    if quantization is None and not args.no_cpu_baseline:
+        cpu = cpu_baseline_e2e(llm, prompts)
+    llm.exit()
+    del llm
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()
+    return res, cpu
+
+
+def cpu_baseline_e2e(llm, prompts, nseq=2, out_tokens=4):
+    """CPU oracle (bf16 F.linear, the reference's own CPU arithmetic) on the first ``nseq`` sequences of the
+    same workload, ``out_tokens`` greedy tokens each, with the same weights copied from the GPU model."""
+    import torch
+    from oracle.model import OracleQwen3, greedy_generate
+    torch.set_num_threads(os.cpu_count() if (os.cpu_count() or 0) <= 64 else 16)
+    cfg = vars(llm.config.hf_config)
+    params = {k: v.data.cpu() for k, v in llm.model_runner.model.named_parameters()}
+    model = OracleQwen3(cfg, params, exact=False)
+    sample = prompts[:nseq]
+    t0 = time.perf_counter()
+    greedy_generate(model, sample, max_tokens=out_tokens, block_size=256)
+    dt = time.perf_counter() - t0
+    return dict(value=round(nseq * out_tokens / dt, 4), unit="tok/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"first {nseq} of 256 sequences of the same workload (prompts {[len(p) for p in sample]} tokens), "
+                       f"{out_tokens} greedy output tokens each, bf16 linears, same weights: {dt:.1f} s of CPU oracle time "
+                       f"(prefill included, as in the metric)")
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -229,36 +322,56 @@ def main():
         print("bench.py needs a GPU (the HIP path has no CPU fallback)", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
-    out = {}
     extra = {}
-    res = bench_decode_attn(args)
+    attn = bench_decode_attn(args)
+    roofline = attn["roofline"]
+    extra["paged_decode_GBps_back_to_back"] = round(attn["value"], 1)
     extra["hbm_probe"] = bench_probes(args)
     if args.workload in ("gemm", "all"):
         extra["w8a16_gemm"] = bench_gemm(args)
-    cpu = None
-    if not args.no_cpu_baseline:
-        cpu = cpu_baseline_decode(res["case"])
+    if args.workload == "decode_attn":
+        cpu = None if args.no_cpu_baseline else cpu_baseline_decode(attn["case"])
+        out = {
+            "metric": "paged-decode HBM GB/s vs peak", "value": round(attn["value"], 1), "unit": "GB/s", "n_gpus": 1,
+            "steps": args.attn_steps, "warmup": 30, "ms_per_step": round(attn["ms_per_step"], 5),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "BASELINE.json configs[1]: paged decode attention microbench, B=%d Hq=32 Hkv=8 "
+                                   "Dh=128 block_size=256 ctx~U[512,4096] pool=2048 blocks" % args.batch,
+                       "total_context_tokens": attn["case"]["total_tokens"]},
+            "roofline": roofline, "cpu_baseline": cpu, "extra": extra}
+        print(json.dumps(out))
+        return
+    del attn
+    torch.cuda.empty_cache()
+    w8, _ = bench_e2e(args, "w8a16")
+    bf, cpu = bench_e2e(args, None)
+    extra["bf16_linears"] = {"tok_s": round(bf["tok_s"], 1), "wall_s": round(bf["wall_s"], 3), "stats": bf["stats"]}
+    extra["w8a16_linears"] = {"tok_s": round(w8["tok_s"], 1), "wall_s": round(w8["wall_s"], 3), "stats": w8["stats"],
+                              "kv_blocks": w8["kv_blocks"]}
+    steps = w8["stats"]["steps"]
     out = {
-        "metric": "paged-decode HBM GB/s vs peak",
-        "value": round(res["value"], 1),
-        "unit": "GB/s",
+        "metric": "output tok/s (Qwen3-8B-shape, 1 GPU); paged-decode HBM GB/s vs peak",
+        "value": round(w8["tok_s"], 1),
+        "unit": "tok/s",
         "n_gpus": 1,
-        "steps": args.steps,
-        "warmup": args.warmup,
-        "ms_per_step": round(res["ms_per_step"], 5),
+        "steps": steps,
+        "warmup": max(1, args.warmup),
+        "ms_per_step": round(1e3 * w8["wall_s"] / max(1, steps), 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
         "data": "synthetic",
-        "config": {"workload": "BASELINE.json configs[1]: paged decode attention microbench, B=%d Hq=32 Hkv=8 Dh=128 "
-                               "block_size=256 ctx~U[512,4096] pool=2048 blocks" % args.batch,
-                   "total_context_tokens": res["case"]["total_tokens"]},
-        "roofline": res["roofline"],
+        "config": {"workload": "BASELINE.json configs[3]: end-to-end Qwen3-8B-shaped decoder, random-init, W8A16 linears "
+                               "(int8 weights, bf16 activations and MFMA), bf16 KV cache, %d sequences, prompts and outputs "
+                               "~U[100,1024] tokens, ignore_eos, greedy, continuous batching, hipGraph decode"
+                               % args.num_seqs,
+                   "total_output_tokens": w8["total_output_tokens"],
+                   "roofline_workload": "BASELINE.json configs[1] paged decode attention microbench"},
+        "roofline": roofline,
         "cpu_baseline": cpu,
+        "extra": extra,
     }
-    if extra:
-        out["extra"] = extra
     print(json.dumps(out))
 
 

@@ -18,22 +18,30 @@ from . import ops as O
 
 
 class OracleQwen3:
-    def __init__(self, cfg: dict, params: dict):
+    def __init__(self, cfg: dict, params: dict, exact: bool = True):
         """``params``: ``{name: tensor}`` with the reference's packed parameter names
-        (``model.layers.N.self_attn.qkv_proj.weight`` ...)."""
+        (``model.layers.N.self_attn.qkv_proj.weight`` ...).  ``exact=False`` runs the linears as the
+        reference does on a CPU (``F.linear`` in bf16, no fp64 copies): used for timing only."""
         self.cfg = dict(cfg)
+        self.exact = exact
         self.p = {k: v.detach().cpu() for k, v in params.items()}
-        self.p64 = {k: v.double() for k, v in self.p.items() if k.endswith("proj.weight") or "embed_tokens" in k
-                    or k.startswith("lm_head")}
+        self.p64 = {}
+        if exact:
+            self.p64 = {k: v.double() for k, v in self.p.items() if k.endswith("proj.weight") or "embed_tokens" in k
+                        or k.startswith("lm_head")}
         c = self.cfg
         self.Hq, self.Hkv, self.Dh = c["num_attention_heads"], c["num_key_value_heads"], c["head_dim"]
         self.eps = c.get("rms_norm_eps", 1e-6)
         self.table = O.rope_table(self.Dh, c.get("max_position_embeddings", 40960), c.get("rope_theta", 1e6))
         self.L = c["num_hidden_layers"]
-        if "lm_head.weight" not in self.p64:
+        if "lm_head.weight" not in self.p:
+            self.p["lm_head.weight"] = self.p["model.embed_tokens.weight"]
+        if exact and "lm_head.weight" not in self.p64:
             self.p64["lm_head.weight"] = self.p64["model.embed_tokens.weight"]
 
     def lin(self, x, name):
+        if not self.exact:
+            return O.linear(x, self.p[name])
         return (x.double() @ self.p64[name].t()).to(x.dtype)
 
     def forward(self, input_ids, positions, caches, slot_mapping, attend):
@@ -67,7 +75,7 @@ class OracleQwen3:
         return x
 
     def logits(self, hidden):
-        return (hidden.double() @ self.p64["lm_head.weight"].t()).to(hidden.dtype)
+        return self.lin(hidden, "lm_head.weight")
 
 
 def greedy_generate(model: OracleQwen3, prompts: list[list[int]], max_tokens: int, block_size: int = 256,
