@@ -39,6 +39,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes per decode-attention launch on the default configs[1] workload, from two rocprofv3 --pmc runs
+# (FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 KiB per dispatch, factors taken from the 1 GiB copy probe), main + merge kernel
+DECODE_ATTN_TRAFFIC_BYTES = int((313290.6 + 2605.8) * 2.0 * 1024 + (5088.1 + 512.0) * 1024)
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
@@ -171,7 +174,8 @@ def bench_decode_attn(args):
     kern_gbps = case["algo_bytes"] / (t["mean_ms"] * 1e-3) / 1e9
     res = dict(ms_per_step=ms_per_step, value=gbps,
                roofline=dict(bound="hbm", achieved=round(kern_gbps, 1), peak=HBM_PEAK_GBPS, unit="GB/s",
-                             frac=round(kern_gbps / HBM_PEAK_GBPS, 4), traffic=None,
+                             frac=round(kern_gbps / HBM_PEAK_GBPS, 4),
+                             traffic=DECODE_ATTN_TRAFFIC_BYTES if args.batch == 64 else None,
                              kernel="paged_decode_kernel<8,false> + paged_decode_merge_kernel",
                              launch_ms_mean=round(t["mean_ms"], 5), launch_ms_median=round(t["median_ms"], 5),
                              launch_ms_min=round(t["min_ms"], 5), algorithmic_bytes=case["algo_bytes"]),
