@@ -108,13 +108,55 @@ struct GemmParams {
 };
 
 // BN x BM output tile per workgroup (BN output channels, BM tokens), 4 waves as WAVES_N x WAVES_M.
-template <int BN, int BM, int WAVES_N, int WAVES_M, bool W8>
-__global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
+// Epilogue shared by the tiled kernels: scale (W8), round once to bf16, 8-byte stores;
+// or fp32 partials when K is split.
+template <int TN, int TM, int WN, int WM, bool W8>
+__device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&acc)[TN][TM], int m0,
+                                              int n0, int wn, int wm, int r, int kg, int split) {
+  // Epilogue.  acc[i][j][v]: token m = m0 + wm*WM + j*32 + r,
+  // channel n = n0 + wn*WN + i*32 + (v/4)*8 + kg*4 + (v%4).
+#pragma unroll
+  for (int j = 0; j < TM; ++j) {
+    const int m = m0 + wm * WM + j * 32 + r;
+    if (m >= p.M) continue;
+#pragma unroll
+    for (int i = 0; i < TN; ++i) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + wn * WN + i * 32 + q * 8 + kg * 4;
+        if (n >= p.N) continue;  // N % 4 == 0, so a group of 4 is all in or all out
+        float o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o[e] = acc[i][j][q * 4 + e];
+        if (p.splits > 1) {
+          float *dst = p.partial + (static_cast<int64_t>(split) * p.M + m) * p.N + n;
+          *reinterpret_cast<float4 *>(dst) = make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+          if (W8) {
+            const float4 s = *reinterpret_cast<const float4 *>(p.scale + n);
+            o[0] *= s.x; o[1] *= s.y; o[2] *= s.z; o[3] *= s.w;
+          }
+          uint2 st;
+          st.x = pack_bf16x2(o[0], o[1]);
+          st.y = pack_bf16x2(o[2], o[3]);
+          *reinterpret_cast<uint2 *>(p.y + static_cast<int64_t>(m) * p.N + n) = st;
+        }
+      }
+    }
+  }
+}
+
+// NBUF = LDS buffers: 2 overlaps the LDS write of tile i+1 with the math of tile i inside one
+// workgroup; 1 halves the LDS footprint so that more workgroups share a CU and overlap each other.
+template <int BN, int BM, int WAVES_N, int WAVES_M, bool W8, int NBUF>
+__global__ __launch_bounds__(256)
+__attribute__((amdgpu_waves_per_eu(BN * BM >= 256 * 256 ? 1 : 2, 8)))  // all but the largest tile: <= 256 registers
+void gemm_kernel(const GemmParams p) {
   static_assert(WAVES_N * WAVES_M == 4, "4 waves");
   constexpr int WN = BN / WAVES_N, WM = BM / WAVES_M;  // per-wave tile
   constexpr int TN = WN / 32, TM = WM / 32;            // 32x32 MFMA tiles per wave
-  __shared__ __attribute__((aligned(16))) unsigned short Ws[2][BN][kLdsK];
-  __shared__ __attribute__((aligned(16))) unsigned short Xs[2][BM][kLdsK];
+  __shared__ __attribute__((aligned(16))) unsigned short Ws[NBUF][BN][kLdsK];
+  __shared__ __attribute__((aligned(16))) unsigned short Xs[NBUF][BM][kLdsK];
 
   // XCD-aware tile order
   const int xcd = blockIdx.x & 7;
@@ -177,46 +219,190 @@ __global__ __launch_bounds__(256) void gemm_kernel(const GemmParams p) {
         for (int j = 0; j < TM; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
     }
-    if (more) {
-      wl.store(Ws[buf ^ 1], tid);
-      xl.store(Xs[buf ^ 1], tid);
+    if (NBUF == 2) {
+      if (more) {
+        wl.store(Ws[buf ^ 1], tid);
+        xl.store(Xs[buf ^ 1], tid);
+      }
+      __syncthreads();
+      buf ^= 1;
+    } else {
+      __syncthreads();  // every wave is done reading the tile
+      if (more) {
+        wl.store(Ws[0], tid);
+        xl.store(Xs[0], tid);
+      }
+      __syncthreads();
     }
-    __syncthreads();
-    buf ^= 1;
   }
 
-  // Epilogue.  acc[i][j][v]: token m = m0 + wm*WM + j*32 + r,
-  // channel n = n0 + wn*WN + i*32 + (v/4)*8 + kg*4 + (v%4).
+  gemm_epilogue<TN, TM, WN, WM, W8>(p, acc, m0, n0, wn, wm, r, kg, split);
+}
+
+// ---------------------------------------------------------------------------
+// Pipelined variant of the tiled kernel for tiles up to 128 x 128 (the mid-size GEMMs of a
+// decode step).  Same tiling and numerics as gemm_kernel; what differs is the schedule:
+//   * two register sets: the global loads of K-tiles t+1 and t+2 are both in flight while tile t
+//     is computed, so a load has two steps to land (loads are unconditional - rows and tiles past
+//     the end are clamped - so that the compiler can count them and never drains the queue);
+//   * the workgroup barrier orders LDS only (lds_barrier), global loads stay in flight across it;
+//   * the int8 -> bf16 conversion and LDS write of tile t+1 are issued in four slices between the
+//     four MFMA groups of tile t, so VALU / LDS work overlaps matrix-core time.
+// Written without lambdas or arrays of loader objects: those end up in scratch memory.
+template <int ROWS, bool W8>
+struct PipeLoader;
+
+template <int ROWS>
+struct PipeLoader<ROWS, false> {  // bf16 rows: 8 lanes x 16 B per row and K-tile
+  static constexpr int kPasses = ROWS / 32;
+  u32x4 r[kPasses];  // native vectors: arrays of HIP's struct uint4 are not promoted to registers here
+  __device__ __forceinline__ void load(const unsigned char *base, int64_t ld_bytes, int row0,
+                                       int rows_total, int k0, int tid) {
 #pragma unroll
-  for (int j = 0; j < TM; ++j) {
-    const int m = m0 + wm * WM + j * 32 + r;
-    if (m >= p.M) continue;
+    for (int p = 0; p < kPasses; ++p) {
+      const int row = min(row0 + p * 32 + (tid >> 3), rows_total - 1);
+      r[p] = *reinterpret_cast<const u32x4 *>(base + row * ld_bytes +
+                                              (static_cast<int64_t>(k0) + (tid & 7) * 8) * 2);
+    }
+  }
+  template <int PART, int NPARTS>
+  __device__ __forceinline__ void store_part(unsigned short (*lds)[kLdsK], int tid) const {
 #pragma unroll
-    for (int i = 0; i < TN; ++i) {
+    for (int p = 0; p < kPasses; ++p)
+      if (p % NPARTS == PART)
+        *reinterpret_cast<u32x4 *>(&lds[p * 32 + (tid >> 3)][(tid & 7) * 8]) = r[p];
+  }
+};
+
+template <int ROWS>
+struct PipeLoader<ROWS, true> {  // int8 rows: 4 lanes x 16 B per row and K-tile
+  static constexpr int kPasses = ROWS / 64;
+  u32x4 r[kPasses];  // native vectors: arrays of HIP's struct uint4 are not promoted to registers here
+  __device__ __forceinline__ void load(const unsigned char *base, int64_t ld_bytes, int row0,
+                                       int rows_total, int k0, int tid) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int n = n0 + wn * WN + i * 32 + q * 8 + kg * 4;
-        if (n >= p.N) continue;  // N % 4 == 0, so a group of 4 is all in or all out
-        float o[4];
+    for (int p = 0; p < kPasses; ++p) {
+      const int row = min(row0 + p * 64 + (tid >> 2), rows_total - 1);
+      r[p] = *reinterpret_cast<const u32x4 *>(base + row * ld_bytes + k0 + (tid & 3) * 16);
+    }
+  }
+  template <int PART, int NPARTS>
+  __device__ __forceinline__ void store_part(unsigned short (*lds)[kLdsK], int tid) const {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) o[e] = acc[i][j][q * 4 + e];
-        if (p.splits > 1) {
-          float *dst = p.partial + (static_cast<int64_t>(split) * p.M + m) * p.N + n;
-          *reinterpret_cast<float4 *>(dst) = make_float4(o[0], o[1], o[2], o[3]);
-        } else {
-          if (W8) {
-            const float4 s = *reinterpret_cast<const float4 *>(p.scale + n);
-            o[0] *= s.x; o[1] *= s.y; o[2] *= s.z; o[3] *= s.w;
-          }
-          uint2 st;
-          st.x = pack_bf16x2(o[0], o[1]);
-          st.y = pack_bf16x2(o[2], o[3]);
-          *reinterpret_cast<uint2 *>(p.y + static_cast<int64_t>(m) * p.N + n) = st;
-        }
+    for (int p = 0; p < kPasses; ++p) {
+      // each pass is cut in two halves so that even a one-pass tile spreads over the slices
+      unsigned short *dst = &lds[p * 64 + (tid >> 2)][(tid & 3) * 16];
+      if ((2 * p) % NPARTS == PART) {
+        const uint2 a = TileLoader<64, true>::cvt4(r[p].x), b = TileLoader<64, true>::cvt4(r[p].y);
+        *reinterpret_cast<uint4 *>(dst) = make_uint4(a.x, a.y, b.x, b.y);
+      }
+      if ((2 * p + 1) % NPARTS == PART) {
+        const uint2 c = TileLoader<64, true>::cvt4(r[p].z), d = TileLoader<64, true>::cvt4(r[p].w);
+        *reinterpret_cast<uint4 *>(dst + 8) = make_uint4(c.x, c.y, d.x, d.y);
       }
     }
   }
+};
+
+#define TLF_PIPE_MFMA(BUF, KS)                                                                    \
+  {                                                                                               \
+    bf16x8 af[TN], bfr[TM];                                                                       \
+    _Pragma("unroll") for (int i = 0; i < TN; ++i) {                                              \
+      Pack16 t;                                                                                   \
+      t.u = *reinterpret_cast<const uint4 *>(&Ws[BUF][wn * WN + i * 32 + r][(KS) * 16 + kg * 8]); \
+      af[i] = t.v;                                                                                \
+    }                                                                                             \
+    _Pragma("unroll") for (int j = 0; j < TM; ++j) {                                              \
+      Pack16 t;                                                                                   \
+      t.u = *reinterpret_cast<const uint4 *>(&Xs[BUF][wm * WM + j * 32 + r][(KS) * 16 + kg * 8]); \
+      bfr[j] = t.v;                                                                               \
+    }                                                                                             \
+    _Pragma("unroll") for (int i = 0; i < TN; ++i)                                                \
+      _Pragma("unroll") for (int j = 0; j < TM; ++j)                                              \
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);   \
+  }
+// one pipeline step: compute buffer BUF while tile (T)+2 is requested into set LD and the already
+// requested tile (T)+1 in set ST is converted and written to the other buffer, slice by slice
+#define TLF_PIPE_STEP(BUF, LDW, LDX, STW, STX, T)                                      \
+  {                                                                                    \
+    const int kl = k_begin + min((T) + 2, nkt - 1) * kBK;                              \
+    LDW.load(p.w, ldw_bytes, n0, p.N, kl, tid);                                        \
+    LDX.load(p.x, p.ldx_bytes, m0, p.M, kl, tid);                                      \
+    TLF_PIPE_MFMA(BUF, 0)                                                              \
+    STW.template store_part<0, 4>(Ws[(BUF) ^ 1], tid);                                 \
+    STX.template store_part<0, 4>(Xs[(BUF) ^ 1], tid);                                 \
+    TLF_PIPE_MFMA(BUF, 1)                                                              \
+    STW.template store_part<1, 4>(Ws[(BUF) ^ 1], tid);                                 \
+    STX.template store_part<1, 4>(Xs[(BUF) ^ 1], tid);                                 \
+    TLF_PIPE_MFMA(BUF, 2)                                                              \
+    STW.template store_part<2, 4>(Ws[(BUF) ^ 1], tid);                                 \
+    STX.template store_part<2, 4>(Xs[(BUF) ^ 1], tid);                                 \
+    TLF_PIPE_MFMA(BUF, 3)                                                              \
+    STW.template store_part<3, 4>(Ws[(BUF) ^ 1], tid);                                 \
+    STX.template store_part<3, 4>(Xs[(BUF) ^ 1], tid);                                 \
+    lds_barrier();                                                                     \
+  }
+
+template <int BN, int BM, int WAVES_N, int WAVES_M, bool W8>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8)))
+void gemm_pipe_kernel(const GemmParams p) {
+  static_assert(WAVES_N * WAVES_M == 4, "4 waves");
+  constexpr int WN = BN / WAVES_N, WM = BM / WAVES_M;
+  constexpr int TN = WN / 32, TM = WM / 32;
+  __shared__ __attribute__((aligned(16))) unsigned short Ws[2][BN][kLdsK];
+  __shared__ __attribute__((aligned(16))) unsigned short Xs[2][BM][kLdsK];
+  const int xcd = blockIdx.x & 7;
+  const int local = blockIdx.x >> 3;
+  const int mt = local % p.m_tiles;
+  const int nt = (local / p.m_tiles) * 8 + xcd;
+  if (nt >= p.n_tiles) return;
+  const int n0 = nt * BN, m0 = mt * BM;
+  const int split = blockIdx.y;
+  const int k_begin = split * p.k_per_split;
+  const int k_end = min(p.K, k_begin + p.k_per_split);
+  const int nkt = (k_end - k_begin) / kBK;
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int wn = wave % WAVES_N, wm = wave / WAVES_N;
+  const int r = lane & 31, kg = lane >> 5;
+  const int64_t ldw_bytes = W8 ? p.K : static_cast<int64_t>(p.K) * 2;
+
+  floatx16 acc[TN][TM];
+#pragma unroll
+  for (int i = 0; i < TN; ++i)
+#pragma unroll
+    for (int j = 0; j < TM; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  PipeLoader<BN, W8> w0, w1;
+  PipeLoader<BM, false> x0, x1;
+  w0.load(p.w, ldw_bytes, n0, p.N, k_begin, tid);
+  x0.load(p.x, p.ldx_bytes, m0, p.M, k_begin, tid);
+  {
+    const int k1 = k_begin + min(1, nkt - 1) * kBK;
+    w1.load(p.w, ldw_bytes, n0, p.N, k1, tid);
+    x1.load(p.x, p.ldx_bytes, m0, p.M, k1, tid);
+  }
+  w0.template store_part<0, 1>(Ws[0], tid);
+  x0.template store_part<0, 1>(Xs[0], tid);
+  lds_barrier();
+  // tile t sits in buffer t & 1; set 1 holds tile t+1 at even t, set 0 at odd t
+  const int pairs = nkt / 2;
+  for (int t = 0; t < 2 * pairs; t += 2) {
+    TLF_PIPE_STEP(0, w0, x0, w1, x1, t)
+    TLF_PIPE_STEP(1, w1, x1, w0, x0, t + 1)
+  }
+  if (nkt & 1) {  // the last tile of an odd count sits in buffer 0 (written by the last odd step)
+    TLF_PIPE_MFMA(0, 0)
+    TLF_PIPE_MFMA(0, 1)
+    TLF_PIPE_MFMA(0, 2)
+    TLF_PIPE_MFMA(0, 3)
+  }
+  gemm_epilogue<TN, TM, WN, WM, W8>(p, acc, m0, n0, wn, wm, r, kg, split);
 }
+#undef TLF_PIPE_STEP
+#undef TLF_PIPE_MFMA
 
 // Sum the split-K partials, apply the channel scale, round once to bf16.
 template <bool W8>
@@ -408,6 +594,8 @@ int launch_skinny(const GemmParams &p, hipStream_t stream) {
 }
 
 struct GemmPlan {
+  bool pipe = false;  // use the pipelined kernel (tiles up to 128 x 128)
+  int nbuf = 2; // LDS buffers
   int bn, bm;   // tile
   int splits;   // split-K factor
   int k_per_split;
@@ -417,7 +605,7 @@ struct GemmPlan {
 // A K-tile step of this kernel costs roughly the same whatever the tile (it is latency bound),
 // so mid-size problems want many small tiles plus a moderate split of K (each split keeps at
 // least 16 K-tiles), and only problems with thousands of tiles use the large MFMA-friendly tiles.
-inline GemmPlan plan_gemm(int M, int N, int K) {
+inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
   GemmPlan g;
   auto tiles = [&](int bn, int bm) { return ((N + bn - 1) / bn) * ((M + bm - 1) / bm); };
   auto pow2_floor = [](int v) { int p = 1; while (p * 2 <= v) p *= 2; return p; };
@@ -430,11 +618,17 @@ inline GemmPlan plan_gemm(int M, int N, int K) {
   } else if (tiles(128, 128) <= 1024) {
     g.bn = 128; g.bm = 128;
     splits = tiles(128, 128) <= 256 ? pow2_floor(512 / tiles(128, 128)) : 1;
-  } else if (tiles(256, 256) >= 256) {
-    g.bn = 256; g.bm = 256;
+    // plenty of tiles: one LDS buffer, so that three workgroups share a CU (measured +5-15 %)
+    if (tiles(128, 128) > 256) g.nbuf = 1;
   } else {
-    g.bn = 128; g.bm = 128;
+    // thousands of tiles: 128 channels x 256 tokens, one LDS buffer, two workgroups per CU
+    // (measured 427 us against 456 us for a 256 x 256 tile on 24576 x 4096 at M = 2048)
+    g.bn = 128; g.bm = 256; g.nbuf = 1;
+    // the bf16-weight variant of that tile does not fit 256 registers: keep the 256 x 256 tile
+    if (!w8) { g.bn = 256; g.bm = 256; g.nbuf = 2; }
   }
+  // small tiles with two LDS buffers run the pipelined schedule (measured 5-25 % faster)
+  g.pipe = g.bn <= 128 && g.bm <= 128 && g.nbuf == 2;
   if (splits > max_split) splits = max_split;
   if (splits > 16) splits = 16;
   if (splits < 1) splits = 1;
@@ -449,8 +643,10 @@ inline GemmPlan plan_gemm(int M, int N, int K) {
 inline bool plan_override(GemmPlan &g, int K) {
   const char *e = getenv("TLF_GEMM_PLAN");
   if (!e) return false;
-  int bn = 0, bm = 0, sp = 0;
-  if (sscanf(e, "%d,%d,%d", &bn, &bm, &sp) != 3) return false;
+  int bn = 0, bm = 0, sp = 0, nb = 2;
+  if (sscanf(e, "%d,%d,%d,%d", &bn, &bm, &sp, &nb) < 3) return false;
+  g.nbuf = nb == 1 ? 1 : 2;
+  g.pipe = nb == 3;
   const int ktiles = K / kBK;
   if (sp < 1) sp = 1;
   if (sp > ktiles) sp = ktiles;
@@ -486,7 +682,7 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
     p.k_per_split = K; p.splits = 1; p.m_tiles = 1; p.n_tiles = 1;
     return launch_skinny<W8>(p, stream);
   }
-  GemmPlan g = plan_gemm(M, N, K);
+  GemmPlan g = plan_gemm(M, N, K, W8);
   plan_override(g, K);
   p.k_per_split = g.k_per_split;
   p.splits = g.splits;
@@ -499,12 +695,28 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
     p.partial = static_cast<float *>(workspace);
   }
   const dim3 grid(((p.n_tiles + 7) / 8) * 8 * p.m_tiles, g.splits);
-#define TLF_TILE(BN_, BM_, WN_, WM_)                                                          \
-  if (g.bn == BN_ && g.bm == BM_) {                                                           \
-    hipLaunchKernelGGL((gemm_kernel<BN_, BM_, WN_, WM_, W8>), grid, dim3(256), 0, stream, p); \
-    launched = true;                                                                          \
+#define TLF_TILE(BN_, BM_, WN_, WM_)                                                               \
+  if (g.bn == BN_ && g.bm == BM_) {                                                                \
+    if (g.nbuf == 1)                                                                               \
+      hipLaunchKernelGGL((gemm_kernel<BN_, BM_, WN_, WM_, W8, 1>), grid, dim3(256), 0, stream, p); \
+    else                                                                                           \
+      hipLaunchKernelGGL((gemm_kernel<BN_, BM_, WN_, WM_, W8, 2>), grid, dim3(256), 0, stream, p); \
+    launched = true;                                                                               \
   }
   bool launched = false;
+  if (g.pipe && g.bm <= 128 && g.bn <= 128) {
+#define TLF_PIPE(BN_, BM_, WN_, WM_)                                                                \
+  if (g.bn == BN_ && g.bm == BM_) {                                                                 \
+    hipLaunchKernelGGL((gemm_pipe_kernel<BN_, BM_, WN_, WM_, W8>), grid, dim3(256), 0, stream, p);  \
+    launched = true;                                                                                \
+  }
+    TLF_PIPE(128, 128, 2, 2)
+    TLF_PIPE(64, 128, 1, 4)
+    TLF_PIPE(128, 64, 4, 1)
+    TLF_PIPE(64, 64, 2, 2)
+#undef TLF_PIPE
+  }
+  if (!launched) {
   TLF_TILE(256, 256, 2, 2)
   TLF_TILE(128, 256, 2, 2)
   TLF_TILE(64, 256, 1, 4)
@@ -513,6 +725,7 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   TLF_TILE(64, 128, 1, 4)
   TLF_TILE(128, 64, 4, 1)
   TLF_TILE(64, 64, 2, 2)
+  }
 #undef TLF_TILE
   if (!launched) return TLF_E_UNSUPPORTED;
   int rc = launch_status();
