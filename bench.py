@@ -50,7 +50,7 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=0, help="timed engine steps of the e2e run (0 = whole job)")
     ap.add_argument("--warmup", type=int, default=1, help="warm-up generate() calls before the timed run")
-    ap.add_argument("--workload", default="e2e", choices=["e2e", "decode_attn", "gemm", "all"])
+    ap.add_argument("--workload", default="e2e", choices=["e2e", "decode_attn", "gemm", "c5", "all"])
     ap.add_argument("--attn-steps", type=int, default=200, help="timed launches of the decode-attention microbench")
     ap.add_argument("--num-seqs", type=int, default=256)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -234,6 +234,39 @@ def bench_gemm(args, ms=(1, 16, 64, 256, 2048)):
     return rows
 
 
+# ----------------------------------------------------------------------------- config 5 (32B shape, fp8 KV, shared prefixes)
+def bench_c5(args):
+    """BASELINE.json configs[4]: Qwen3-32B-shaped decoder, W8A16 linears, e4m3 KV cache with per-head scales,
+    32 sequences with prompts ~U[2048, 8192], half of them sharing a 1024-token prefix held in cached blocks
+    (a first generate() of one prefix-only request fills those blocks), 256 greedy output tokens each."""
+    import torch
+    from random import randint, seed
+    from tinyllmforge_amd import LLM, SamplingParams
+    seed(0)
+    shared = [randint(0, 10000) for _ in range(1024)]
+    prompts = []
+    for i in range(32):
+        n = randint(2048, 8192)
+        body = [randint(0, 10000) for _ in range(n)]
+        prompts.append(shared + body[1024:] if i % 2 == 0 else body)
+    llm = LLM("qwen3-32b", enforce_eager=False, max_model_len=8704, max_num_batched_tokens=16384, max_num_seqs=32,
+              quantization="w8a16", kv_cache_dtype="fp8_e4m3", gpu_memory_utilization=0.6, seed=0)
+    sp = SamplingParams(temperature=0.0, ignore_eos=True, max_tokens=256)
+    llm.generate([shared + [1, 2, 3]], SamplingParams(temperature=0.0, max_tokens=2, ignore_eos=True))   # warm-up + prefix fill
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    llm.generate(prompts, sp)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    st = llm.last_stats
+    res = dict(tok_s=round(32 * 256 / wall, 1), wall_s=round(wall, 3), prompt_tokens=sum(len(p) for p in prompts),
+               prefill_s=round(st["prefill_time"], 3), decode_s=round(st["decode_time"], 3),
+               decode_ms_per_step=round(1e3 * st["decode_time"] / max(1, st["decode_steps"]), 3),
+               kv_blocks=llm.config.num_kvcache_blocks, kv_dtype="fp8_e4m3")
+    llm.exit()
+    return res
+
+
 # ----------------------------------------------------------------------------- config 4 (end to end)
 def e2e_workload(num_seqs=256):
     """The reference's bench.py recipe (pure-python ``random``: platform independent)."""
@@ -347,6 +380,11 @@ def main():
         return
     del attn
     torch.cuda.empty_cache()
+    if args.workload in ("c5", "all"):
+        extra["config5_qwen3_32b_fp8kv"] = bench_c5(args)
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
     w8, _ = bench_e2e(args, "w8a16")
     bf, cpu = bench_e2e(args, None)
     extra["bf16_linears"] = {"tok_s": round(bf["tok_s"], 1), "wall_s": round(bf["wall_s"], 3), "stats": bf["stats"]}

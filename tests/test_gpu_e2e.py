@@ -171,3 +171,34 @@ def test_temperature_sampling_runs_and_respects_greedy_rows():
     assert mixed[0]["token_ids"] == greedy
     assert all(0 <= t < 1024 for t in mixed[1]["token_ids"])
     llm.exit()
+
+
+def test_fp8_kv_cache_with_shared_prefix_end_to_end():
+    """Config-5 style run at small scale: W8A16 linears, e4m3 KV cache, half of the prompts share a
+    512-token prefix that is held in cached blocks (second wave of requests hits it and takes the
+    paged-prefill path, reading e4m3 rows back).  The e4m3 cache must track the bf16 cache closely."""
+    from tinyllmforge_amd import LLM, SamplingParams
+    g = torch.Generator().manual_seed(7)
+    shared = torch.randint(0, 5000, (512,), generator=g).tolist()
+    prompts = []
+    for i in range(6):
+        tail = torch.randint(0, 5000, (100 + 37 * i,), generator=g).tolist()
+        prompts.append((shared + tail) if i % 2 == 0 else torch.randint(0, 5000, (300 + 50 * i,), generator=g).tolist())
+    sp = SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True)
+    outs = {}
+    for kv in ("bf16", "fp8_e4m3"):
+        llm = LLM("qwen3-0.6b", max_model_len=2048, max_num_batched_tokens=4096, max_num_seqs=8, num_kvcache_blocks=40,
+                  enforce_eager=False, seed=0, quantization="w8a16", kv_cache_dtype=kv)
+        first = llm.generate(prompts[:2], sp)                       # fills the prefix blocks
+        bm = llm.scheduler.block_manager
+        assert len(bm.hash_to_block_id) >= 2
+        rest = llm.generate(prompts, sp)                            # prompts 0, 2, 4 hit the shared prefix
+        assert [len(o["token_ids"]) for o in rest] == [12] * 6
+        # same request, now with its prefix served from cached blocks (paged prefill path): the first
+        # token must agree (later ones may part at near-ties of this random-weight model)
+        assert rest[0]["token_ids"][0] == first[0]["token_ids"][0]
+        outs[kv] = [o["token_ids"] for o in rest]
+        assert llm.model_runner.kv_cache.dtype == (torch.bfloat16 if kv == "bf16" else torch.float8_e4m3fn)
+        llm.exit()
+    agree = sum(a[0] == b[0] for a, b in zip(outs["bf16"], outs["fp8_e4m3"]))
+    assert agree >= 4, f"first tokens with e4m3 KV agree with bf16 KV on only {agree} of 6 sequences"

@@ -575,6 +575,10 @@ int launch_skinny(const GemmParams &p, hipStream_t stream) {
   int tn = 1;
   if (tiles16 >= 4 * 512) tn = 4;
   else if (tiles16 >= 2 * 512) tn = 2;
+  if (const char *e = getenv("TLF_GEMM_SKINNY_TN")) {  // tuning override
+    const int v = atoi(e);
+    if (v == 1 || v == 2 || v == 4) tn = v;
+  }
   const dim3 grid((tiles16 + tn - 1) / tn);
 #define TLF_SK(MT_, TN_) \
   hipLaunchKernelGGL((skinny_gemm_kernel<MT_, TN_, W8>), grid, dim3(512), 0, stream, p)
