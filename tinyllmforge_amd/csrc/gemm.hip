@@ -9,17 +9,14 @@
 // the per-channel scale is a per-register constant and the bf16 result is
 // written as 8-byte pieces of a y row.
 //
-//   global --128-bit loads--> registers --(int8 -> bf16, exact)--> LDS (padded rows)
-//   LDS --ds_read_b128--> v_mfma_f32_32x32x16_bf16, fp32 accumulators
-//
-// LDS is double buffered: while the matrix cores work on K-tile i, the loads of
-// K-tile i+1 are in flight to registers, then converted and written to the
-// other buffer; one barrier per K-tile.
+// Two kernels: a tiled one whose K-tiles travel global -> LDS without passing
+// through registers (gemm_dlds_kernel, more than 16 tokens) and a skinny one
+// that streams W straight into MFMA operand registers (skinny_gemm_kernel).
 //
 // Tile order is XCD aware: hardware deals workgroups round-robin to the 8 XCDs
 // (each with a private L2), so workgroup b belongs to XCD b % 8.  Each XCD is
-// given whole columns of N-tiles and walks the M-tiles of a column first, so
-// the workgroups that share an L2 share W panels and step through K together.
+// given whole columns of N-tiles, so the workgroups that share an L2 share W
+// and x panels and step through K together.
 #include <stdio.h>
 #include <stdlib.h>
 
@@ -28,71 +25,16 @@
 namespace tlf {
 
 constexpr int kBK = 64;           // K elements per LDS tile
-constexpr int kLdsK = kBK + 8;    // padded LDS row: 144 B
 constexpr int kSkinnyMaxM = 16;   // at or below this many tokens the skinny kernel runs
 
-template <int ROWS, bool W8>
-struct TileLoader;
-
-// bf16 source rows: 128 B per row per K-tile = 8 lanes x 16 B.
-template <int ROWS>
-struct TileLoader<ROWS, false> {
-  static constexpr int kPasses = ROWS / 32;  // 256 threads cover 32 rows per pass
-  uint4 r[kPasses];
-  __device__ __forceinline__ void load(const unsigned char *base, int64_t ld_bytes, int row0,
-                                       int rows_total, int k0, int tid) {
-    const int c = tid & 7;
-#pragma unroll
-    for (int p = 0; p < kPasses; ++p) {
-      const int row = p * 32 + (tid >> 3);
-      r[p] = make_uint4(0, 0, 0, 0);
-      if (row0 + row < rows_total)
-        r[p] = *reinterpret_cast<const uint4 *>(base + (row0 + row) * ld_bytes +
-                                                (static_cast<int64_t>(k0) + c * 8) * 2);
-    }
-  }
-  __device__ __forceinline__ void store(unsigned short (*lds)[kLdsK], int tid) const {
-    const int c = tid & 7;
-#pragma unroll
-    for (int p = 0; p < kPasses; ++p)
-      *reinterpret_cast<uint4 *>(&lds[p * 32 + (tid >> 3)][c * 8]) = r[p];
-  }
-};
-
-// int8 source rows: 64 B per row per K-tile = 4 lanes x 16 B, converted to bf16 on the way.
-template <int ROWS>
-struct TileLoader<ROWS, true> {
-  static constexpr int kPasses = ROWS / 64;
-  uint4 r[kPasses];
-  __device__ __forceinline__ void load(const unsigned char *base, int64_t ld_bytes, int row0,
-                                       int rows_total, int k0, int tid) {
-    const int c = tid & 3;
-#pragma unroll
-    for (int p = 0; p < kPasses; ++p) {
-      const int row = p * 64 + (tid >> 2);
-      r[p] = make_uint4(0, 0, 0, 0);
-      if (row0 + row < rows_total)
-        r[p] = *reinterpret_cast<const uint4 *>(base + (row0 + row) * ld_bytes + k0 + c * 16);
-    }
-  }
-  static __device__ __forceinline__ uint2 cvt4(unsigned int w) {
-    const float f0 = static_cast<float>(static_cast<signed char>(w & 0xff));
-    const float f1 = static_cast<float>(static_cast<signed char>((w >> 8) & 0xff));
-    const float f2 = static_cast<float>(static_cast<signed char>((w >> 16) & 0xff));
-    const float f3 = static_cast<float>(static_cast<signed char>(w >> 24));
-    return make_uint2(pack_bf16x2(f0, f1), pack_bf16x2(f2, f3));
-  }
-  __device__ __forceinline__ void store(unsigned short (*lds)[kLdsK], int tid) const {
-    const int c = tid & 3;
-#pragma unroll
-    for (int p = 0; p < kPasses; ++p) {
-      const uint2 a = cvt4(r[p].x), b = cvt4(r[p].y), cc = cvt4(r[p].z), d = cvt4(r[p].w);
-      unsigned short *dst = &lds[p * 64 + (tid >> 2)][c * 16];
-      *reinterpret_cast<uint4 *>(dst) = make_uint4(a.x, a.y, b.x, b.y);
-      *reinterpret_cast<uint4 *>(dst + 8) = make_uint4(cc.x, cc.y, d.x, d.y);
-    }
-  }
-};
+// four int8 (one dword) -> four bf16, exact
+__device__ __forceinline__ uint2 cvt4_i8_bf16(unsigned int w) {
+  const float f0 = static_cast<float>(static_cast<signed char>(w & 0xff));
+  const float f1 = static_cast<float>(static_cast<signed char>((w >> 8) & 0xff));
+  const float f2 = static_cast<float>(static_cast<signed char>((w >> 16) & 0xff));
+  const float f3 = static_cast<float>(static_cast<signed char>(w >> 24));
+  return make_uint2(pack_bf16x2(f0, f1), pack_bf16x2(f2, f3));
+}
 
 struct GemmParams {
   const unsigned char *x;
@@ -105,6 +47,7 @@ struct GemmParams {
   int32_t k_per_split;
   int32_t splits;
   int32_t m_tiles, n_tiles;
+  int32_t group_n;  // N-tile columns walked together by one XCD (direct-to-LDS kernel)
 };
 
 // BN x BM output tile per workgroup (BN output channels, BM tokens), 4 waves as WAVES_N x WAVES_M.
@@ -146,215 +89,175 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
   }
 }
 
-// NBUF = LDS buffers: 2 overlaps the LDS write of tile i+1 with the math of tile i inside one
-// workgroup; 1 halves the LDS footprint so that more workgroups share a CU and overlap each other.
-template <int BN, int BM, int WAVES_N, int WAVES_M, bool W8, int NBUF>
-__global__ __launch_bounds__(256)
-__attribute__((amdgpu_waves_per_eu(BN * BM >= 256 * 256 ? 1 : 2, 8)))  // all but the largest tile: <= 256 registers
-void gemm_kernel(const GemmParams p) {
-  static_assert(WAVES_N * WAVES_M == 4, "4 waves");
-  constexpr int WN = BN / WAVES_N, WM = BM / WAVES_M;  // per-wave tile
-  constexpr int TN = WN / 32, TM = WM / 32;            // 32x32 MFMA tiles per wave
-  __shared__ __attribute__((aligned(16))) unsigned short Ws[NBUF][BN][kLdsK];
-  __shared__ __attribute__((aligned(16))) unsigned short Xs[NBUF][BM][kLdsK];
-
-  // XCD-aware tile order
-  const int xcd = blockIdx.x & 7;
-  const int local = blockIdx.x >> 3;
-  const int mt = local % p.m_tiles;
-  const int nt = (local / p.m_tiles) * 8 + xcd;
-  if (nt >= p.n_tiles) return;  // uniform per workgroup
-  const int n0 = nt * BN, m0 = mt * BM;
-  const int split = blockIdx.y;
-  const int k_begin = split * p.k_per_split;
-  const int k_end = min(p.K, k_begin + p.k_per_split);
-
-  const int tid = threadIdx.x;
-  const int wave = tid >> 6, lane = tid & 63;
-  const int wn = wave % WAVES_N, wm = wave / WAVES_N;
-  const int r = lane & 31, kg = lane >> 5;
-
-  floatx16 acc[TN][TM];
-#pragma unroll
-  for (int i = 0; i < TN; ++i)
-#pragma unroll
-    for (int j = 0; j < TM; ++j)
-#pragma unroll
-      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-
-  TileLoader<BN, W8> wl;
-  TileLoader<BM, false> xl;
-  const int64_t ldw_bytes = W8 ? p.K : static_cast<int64_t>(p.K) * 2;
-  wl.load(p.w, ldw_bytes, n0, p.N, k_begin, tid);
-  xl.load(p.x, p.ldx_bytes, m0, p.M, k_begin, tid);
-  wl.store(Ws[0], tid);
-  xl.store(Xs[0], tid);
-  __syncthreads();
-
-  int buf = 0;
-  for (int k0 = k_begin; k0 < k_end; k0 += kBK) {
-    const bool more = k0 + kBK < k_end;
-    if (more) {
-      wl.load(p.w, ldw_bytes, n0, p.N, k0 + kBK, tid);
-      xl.load(p.x, p.ldx_bytes, m0, p.M, k0 + kBK, tid);
-    }
-#pragma unroll
-    for (int ks = 0; ks < kBK / 16; ++ks) {
-      bf16x8 af[TN], bfr[TM];
-#pragma unroll
-      for (int i = 0; i < TN; ++i) {
-        Pack16 t;
-        t.u = *reinterpret_cast<const uint4 *>(&Ws[buf][wn * WN + i * 32 + r][ks * 16 + kg * 8]);
-        af[i] = t.v;
-      }
-#pragma unroll
-      for (int j = 0; j < TM; ++j) {
-        Pack16 t;
-        t.u = *reinterpret_cast<const uint4 *>(&Xs[buf][wm * WM + j * 32 + r][ks * 16 + kg * 8]);
-        bfr[j] = t.v;
-      }
-#pragma unroll
-      for (int i = 0; i < TN; ++i)
-#pragma unroll
-        for (int j = 0; j < TM; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
-    }
-    if (NBUF == 2) {
-      if (more) {
-        wl.store(Ws[buf ^ 1], tid);
-        xl.store(Xs[buf ^ 1], tid);
-      }
-      __syncthreads();
-      buf ^= 1;
-    } else {
-      __syncthreads();  // every wave is done reading the tile
-      if (more) {
-        wl.store(Ws[0], tid);
-        xl.store(Xs[0], tid);
-      }
-      __syncthreads();
-    }
-  }
-
-  gemm_epilogue<TN, TM, WN, WM, W8>(p, acc, m0, n0, wn, wm, r, kg, split);
-}
-
 // ---------------------------------------------------------------------------
-// Pipelined variant of the tiled kernel for tiles up to 128 x 128 (the mid-size GEMMs of a
-// decode step).  Same tiling and numerics as gemm_kernel; what differs is the schedule:
-//   * two register sets: the global loads of K-tiles t+1 and t+2 are both in flight while tile t
-//     is computed, so a load has two steps to land (loads are unconditional - rows and tiles past
-//     the end are clamped - so that the compiler can count them and never drains the queue);
-//   * the workgroup barrier orders LDS only (lds_barrier), global loads stay in flight across it;
-//   * the int8 -> bf16 conversion and LDS write of tile t+1 are issued in four slices between the
-//     four MFMA groups of tile t, so VALU / LDS work overlaps matrix-core time.
-// Written without lambdas or arrays of loader objects: those end up in scratch memory.
-template <int ROWS, bool W8>
-struct PipeLoader;
+// Tiled kernel: global_load_lds_dwordx4 copies each lane's 16 bytes from global memory
+// straight into LDS (the wave's 64 pieces land contiguously at a wave-uniform LDS base), so a K-tile
+// costs no staging registers, no ds_write and - for int8 weights - half the LDS bytes: W stays
+// int8 in LDS and is converted to bf16 after the fragment read.  Three LDS stages, each its own
+// __shared__ object (the compiler then tracks which outstanding copies a ds_read has to wait
+// for per object): while tile t is computed, the copies of tiles t+1 and t+2 are in flight.
+//
+// LDS rows are unpadded (a wave's copy is contiguous), conflicts are avoided by an XOR swizzle of
+// the 16-byte pieces instead: piece c of a 128-byte bf16 row R sits at position c ^ ((R>>1)&7),
+// piece c of a 64-byte int8 row at c ^ ((R>>2)&3); the lane that fills a position picks the
+// matching global piece.  Any 16 consecutive rows then cover all 64 banks once per ds_read_b128.
+//
+// int8 weights: lane (r, kg) reads 16 consecutive K values of channel r with one ds_read_b128 and
+// feeds them to two MFMAs; the K index inside an MFMA is only a summation label, so the x operand
+// of those two MFMAs is read with the same labelling (pieces 2c and 2c+1 of the x row).
+#define TLF_GPTR(p) ((const __attribute__((address_space(1))) void *)(p))
+#define TLF_LPTR(p) ((__attribute__((address_space(3))) void *)(p))
+// Workgroup barrier for the copy pipeline: wait until at most N of this wave's copies are still
+// in flight and its LDS reads have returned, then s_barrier.  Written as one asm block: a
+// workgroup-scope release fence would make the compiler wait for every outstanding copy
+// (they count as LDS writes), which is exactly the wait the pipeline must not do.
+#define TLF_DL_BARRIER(N) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory")
 
-template <int ROWS>
-struct PipeLoader<ROWS, false> {  // bf16 rows: 8 lanes x 16 B per row and K-tile
-  static constexpr int kPasses = ROWS / 32;
-  u32x4 r[kPasses];  // native vectors: arrays of HIP's struct uint4 are not promoted to registers here
-  __device__ __forceinline__ void load(const unsigned char *base, int64_t ld_bytes, int row0,
-                                       int rows_total, int k0, int tid) {
-#pragma unroll
-    for (int p = 0; p < kPasses; ++p) {
-      const int row = min(row0 + p * 32 + (tid >> 3), rows_total - 1);
-      r[p] = *reinterpret_cast<const u32x4 *>(base + row * ld_bytes +
-                                              (static_cast<int64_t>(k0) + (tid & 7) * 8) * 2);
-    }
-  }
-  template <int PART, int NPARTS>
-  __device__ __forceinline__ void store_part(unsigned short (*lds)[kLdsK], int tid) const {
-#pragma unroll
-    for (int p = 0; p < kPasses; ++p)
-      if (p % NPARTS == PART)
-        *reinterpret_cast<u32x4 *>(&lds[p * 32 + (tid >> 3)][(tid & 7) * 8]) = r[p];
-  }
-};
+// The copies are issued from inline asm so that the compiler does not see them: it cannot tell
+// which LDS object a copy writes, and would otherwise wait for every outstanding copy (and for
+// every outstanding LDS read) before each ds_read.  Ordering is explicit instead: TLF_DL_BARRIER.
+// m0 (the LDS base of a copy) is a reserved register that nothing else in this kernel uses:
+// LDS reads and writes need no m0 on this ISA.
+#define TLF_DL_COPY(VOFF, SBASE, LDS)                                                     \
+  asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(VOFF), \
+               "s"(SBASE), "s"(LDS)                                                       \
+               : "memory")
+#define TLF_DL_LDSADDR(P) static_cast<unsigned int>(reinterpret_cast<uintptr_t>(TLF_LPTR(P)))
 
-template <int ROWS>
-struct PipeLoader<ROWS, true> {  // int8 rows: 4 lanes x 16 B per row and K-tile
-  static constexpr int kPasses = ROWS / 64;
-  u32x4 r[kPasses];  // native vectors: arrays of HIP's struct uint4 are not promoted to registers here
-  __device__ __forceinline__ void load(const unsigned char *base, int64_t ld_bytes, int row0,
-                                       int rows_total, int k0, int tid) {
-#pragma unroll
-    for (int p = 0; p < kPasses; ++p) {
-      const int row = min(row0 + p * 64 + (tid >> 2), rows_total - 1);
-      r[p] = *reinterpret_cast<const u32x4 *>(base + row * ld_bytes + k0 + (tid & 3) * 16);
-    }
-  }
-  template <int PART, int NPARTS>
-  __device__ __forceinline__ void store_part(unsigned short (*lds)[kLdsK], int tid) const {
-#pragma unroll
-    for (int p = 0; p < kPasses; ++p) {
-      // each pass is cut in two halves so that even a one-pass tile spreads over the slices
-      unsigned short *dst = &lds[p * 64 + (tid >> 2)][(tid & 3) * 16];
-      if ((2 * p) % NPARTS == PART) {
-        const uint2 a = TileLoader<64, true>::cvt4(r[p].x), b = TileLoader<64, true>::cvt4(r[p].y);
-        *reinterpret_cast<uint4 *>(dst) = make_uint4(a.x, a.y, b.x, b.y);
-      }
-      if ((2 * p + 1) % NPARTS == PART) {
-        const uint2 c = TileLoader<64, true>::cvt4(r[p].z), d = TileLoader<64, true>::cvt4(r[p].w);
-        *reinterpret_cast<uint4 *>(dst + 8) = make_uint4(c.x, c.y, d.x, d.y);
-      }
-    }
-  }
-};
-
-#define TLF_PIPE_MFMA(BUF, KS)                                                                    \
+// Copy setup for one step: global bases and LDS bases of tile T's destination stage.
+#define TLF_DL_ISSUE_SETUP(XS, WS, T)                                                             \
+  const int kt_ = min((T), nkt - 1);                                                              \
+  const unsigned char *xg_ = xbase + static_cast<int64_t>(kt_) * (kBK * 2);                       \
+  const unsigned char *wg_ = wbase + static_cast<int64_t>(kt_) * kWRow;                           \
+  const unsigned int xl_ = TLF_DL_LDSADDR(XS) + wave_u * 1024, wl_ = TLF_DL_LDSADDR(WS) + wave_u * 1024;
+// Slice PART of 4 of the copies.  The copies are spread over the step, between the MFMA groups:
+// issued back to back, the workgroup's copies queue up in the texture-address unit and every
+// wave sits in that queue with nothing on the matrix cores.
+#define TLF_DL_ISSUE_PART(PART)                                                                   \
   {                                                                                               \
-    bf16x8 af[TN], bfr[TM];                                                                       \
-    _Pragma("unroll") for (int i = 0; i < TN; ++i) {                                              \
-      Pack16 t;                                                                                   \
-      t.u = *reinterpret_cast<const uint4 *>(&Ws[BUF][wn * WN + i * 32 + r][(KS) * 16 + kg * 8]); \
-      af[i] = t.v;                                                                                \
-    }                                                                                             \
-    _Pragma("unroll") for (int j = 0; j < TM; ++j) {                                              \
-      Pack16 t;                                                                                   \
-      t.u = *reinterpret_cast<const uint4 *>(&Xs[BUF][wm * WM + j * 32 + r][(KS) * 16 + kg * 8]); \
-      bfr[j] = t.v;                                                                               \
-    }                                                                                             \
-    _Pragma("unroll") for (int i = 0; i < TN; ++i)                                                \
-      _Pragma("unroll") for (int j = 0; j < TM; ++j)                                              \
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);   \
+    _Pragma("unroll") for (int q = 0; q < XP; ++q)                                                \
+      if (q % 4 == (PART)) TLF_DL_COPY(xoff[q], xg_, xl_ + q * kPass);                            \
+    _Pragma("unroll") for (int q = 0; q < WP; ++q)                                                \
+      if ((q + XP) % 4 == (PART)) TLF_DL_COPY(woff[q], wg_, wl_ + q * kPass);                     \
   }
-// one pipeline step: compute buffer BUF while tile (T)+2 is requested into set LD and the already
-// requested tile (T)+1 in set ST is converted and written to the other buffer, slice by slice
-#define TLF_PIPE_STEP(BUF, LDW, LDX, STW, STX, T)                                      \
-  {                                                                                    \
-    const int kl = k_begin + min((T) + 2, nkt - 1) * kBK;                              \
-    LDW.load(p.w, ldw_bytes, n0, p.N, kl, tid);                                        \
-    LDX.load(p.x, p.ldx_bytes, m0, p.M, kl, tid);                                      \
-    TLF_PIPE_MFMA(BUF, 0)                                                              \
-    STW.template store_part<0, 4>(Ws[(BUF) ^ 1], tid);                                 \
-    STX.template store_part<0, 4>(Xs[(BUF) ^ 1], tid);                                 \
-    TLF_PIPE_MFMA(BUF, 1)                                                              \
-    STW.template store_part<1, 4>(Ws[(BUF) ^ 1], tid);                                 \
-    STX.template store_part<1, 4>(Xs[(BUF) ^ 1], tid);                                 \
-    TLF_PIPE_MFMA(BUF, 2)                                                              \
-    STW.template store_part<2, 4>(Ws[(BUF) ^ 1], tid);                                 \
-    STX.template store_part<2, 4>(Xs[(BUF) ^ 1], tid);                                 \
-    TLF_PIPE_MFMA(BUF, 3)                                                              \
-    STW.template store_part<3, 4>(Ws[(BUF) ^ 1], tid);                                 \
-    STX.template store_part<3, 4>(Xs[(BUF) ^ 1], tid);                                 \
-    lds_barrier();                                                                     \
+#define TLF_DL_ISSUE(XS, WS, T)        \
+  {                                    \
+    TLF_DL_ISSUE_SETUP(XS, WS, T)      \
+    TLF_DL_ISSUE_PART(0)               \
+    TLF_DL_ISSUE_PART(1)               \
+    TLF_DL_ISSUE_PART(2)               \
+    TLF_DL_ISSUE_PART(3)               \
   }
 
-template <int BN, int BM, int WAVES_N, int WAVES_M, bool W8>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 8)))
-void gemm_pipe_kernel(const GemmParams p) {
-  static_assert(WAVES_N * WAVES_M == 4, "4 waves");
+// Copy slices issued after MFMA group G (0..3) of a step.  Three stages: one slice per group.
+// Two stages: the copy has to land within the step, so everything goes out in its first half.
+#define TLF_DL_AFTER_GROUP(G)                          \
+  if constexpr (NS == 3) {                             \
+    if ((G) == 0) TLF_DL_ISSUE_PART(0)                 \
+    if ((G) == 1) TLF_DL_ISSUE_PART(1)                 \
+    if ((G) == 2) TLF_DL_ISSUE_PART(2)                 \
+    if ((G) == 3) TLF_DL_ISSUE_PART(3)                 \
+  } else {                                             \
+    if ((G) == 0) { TLF_DL_ISSUE_PART(0) TLF_DL_ISSUE_PART(1) } \
+    if ((G) == 1) { TLF_DL_ISSUE_PART(2) TLF_DL_ISSUE_PART(3) } \
+  }
+// Compute on stage (XS, WS); the four copy slices of the step go between its MFMA groups.
+#define TLF_DL_COMPUTE(XS, WS)                                                                    \
+  if constexpr (W8) {                                                                             \
+    _Pragma("unroll") for (int ksp = 0; ksp < 2; ++ksp) {                                         \
+      bf16x8 af[TN][2], bfr[TM][2];                                                               \
+      _Pragma("unroll") for (int i = 0; i < TN; ++i) {                                            \
+        const u32x4 raw = *reinterpret_cast<const u32x4 *>(WS + wrow + i * (32 * 64) + wq[ksp]);  \
+        const uint2 a = cvt4_i8_bf16(raw.x), b = cvt4_i8_bf16(raw.y); \
+        const uint2 c = cvt4_i8_bf16(raw.z), d = cvt4_i8_bf16(raw.w); \
+        Pack16 t;                                                                                 \
+        t.u = make_uint4(a.x, a.y, b.x, b.y);                                                     \
+        af[i][0] = t.v;                                                                           \
+        t.u = make_uint4(c.x, c.y, d.x, d.y);                                                     \
+        af[i][1] = t.v;                                                                           \
+      }                                                                                           \
+      _Pragma("unroll") for (int h = 0; h < 2; ++h)                                               \
+        _Pragma("unroll") for (int j = 0; j < TM; ++j) {                                          \
+          Pack16 t;                                                                               \
+          t.u = *reinterpret_cast<const uint4 *>(XS + xrow + j * (32 * 128) + xq[ksp * 2 + h]);   \
+          bfr[j][h] = t.v;                                                                        \
+        }                                                                                         \
+      _Pragma("unroll") for (int h = 0; h < 2; ++h) {                                             \
+        _Pragma("unroll") for (int i = 0; i < TN; ++i)                                            \
+          _Pragma("unroll") for (int j = 0; j < TM; ++j)                                          \
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i][h], bfr[j][h], acc[i][j], 0, 0, 0); \
+        TLF_DL_AFTER_GROUP(ksp * 2 + h)                                                           \
+      }                                                                                           \
+    }                                                                                             \
+  } else {                                                                                        \
+    _Pragma("unroll") for (int ks = 0; ks < 4; ++ks) {                                            \
+      bf16x8 af[TN], bfr[TM];                                                                     \
+      _Pragma("unroll") for (int i = 0; i < TN; ++i) {                                            \
+        Pack16 t;                                                                                 \
+        t.u = *reinterpret_cast<const uint4 *>(WS + wrow + i * (32 * 128) + xq[ks]);              \
+        af[i] = t.v;                                                                              \
+      }                                                                                           \
+      _Pragma("unroll") for (int j = 0; j < TM; ++j) {                                            \
+        Pack16 t;                                                                                 \
+        t.u = *reinterpret_cast<const uint4 *>(XS + xrow + j * (32 * 128) + xq[ks]);              \
+        bfr[j] = t.v;                                                                             \
+      }                                                                                           \
+      _Pragma("unroll") for (int i = 0; i < TN; ++i)                                              \
+        _Pragma("unroll") for (int j = 0; j < TM; ++j)                                            \
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0); \
+      TLF_DL_AFTER_GROUP(ks)                                                                      \
+    }                                                                                             \
+  }
+
+// One step: tile T sits in stage (XS, WS).  Own copies of tile T have landed once at most one
+// later tile (kLoads copies) is outstanding; the barrier then makes every wave's copies visible
+// and says that every wave is done with the stage tile T+2 goes to (it held tile T-1).
+#define TLF_DL_STEP(XS, WS, XS_NEXT2, WS_NEXT2, T) \
+  {                                                \
+    TLF_DL_BARRIER(kLoads);                        \
+    TLF_DL_ISSUE_SETUP(XS_NEXT2, WS_NEXT2, (T) + 2) \
+    TLF_DL_COMPUTE(XS, WS)                         \
+  }
+// Two-stage form: the copy of tile T+1 is issued right after the barrier of step T into the stage
+// tile T-1 was read from, and has the whole step to land (an L2 hit takes a few hundred cycles,
+// a step a thousand or more).  Half the LDS of the three-stage form, so more workgroups per CU.
+#define TLF_DL_STEP2(XS, WS, XS_NEXT, WS_NEXT, T) \
+  {                                               \
+    TLF_DL_BARRIER(0);                            \
+    TLF_DL_ISSUE_SETUP(XS_NEXT, WS_NEXT, (T) + 1) \
+    TLF_DL_COMPUTE(XS, WS)                        \
+  }
+
+// NS = LDS stages (2 or 3), OCC = waves per SIMD the register budget is cut for.
+template <int BN, int BM, int WAVES_N, int WAVES_M, bool W8, int NS, int OCC>
+__global__ __launch_bounds__(WAVES_N * WAVES_M * 64) __attribute__((amdgpu_waves_per_eu(OCC, 8)))
+void gemm_dlds_kernel(const GemmParams p) {
+  static_assert(NS == 2 || NS == 3, "2 or 3 stages");
+  constexpr int NW = WAVES_N * WAVES_M;       // 4 waves, or 8 so that two waves share each SIMD
+  static_assert(NW == 4 || NW == 8, "4 or 8 waves");  // 8: two waves share each SIMD (not faster in the sweeps)
   constexpr int WN = BN / WAVES_N, WM = BM / WAVES_M;
   constexpr int TN = WN / 32, TM = WM / 32;
-  __shared__ __attribute__((aligned(16))) unsigned short Ws[2][BN][kLdsK];
-  __shared__ __attribute__((aligned(16))) unsigned short Xs[2][BM][kLdsK];
+  constexpr int kWRow = W8 ? kBK : kBK * 2;   // bytes of one W row in a K-tile
+  constexpr int kPass = NW * 1024;            // bytes one copy instruction moves per workgroup
+  constexpr int XP = BM * 128 / kPass;        // copies per lane and stage: x
+  constexpr int WP = BN * kWRow / kPass;      // ... and W
+  constexpr int kLoads = XP + WP;
+  static_assert(XP >= 1 && WP >= 1 && TN >= 1 && TM >= 1, "tile too small");
+  static_assert(NS * (BM * 128 + BN * kWRow) <= 160 * 1024, "the stages must fit LDS");
+  static_assert(kLoads <= 31, "vmcnt range");
+  __shared__ __attribute__((aligned(1024))) unsigned char Xs0[BM * 128], Xs1[BM * 128], Xs2[BM * 128];
+  __shared__ __attribute__((aligned(1024))) unsigned char Ws0[BN * kWRow], Ws1[BN * kWRow], Ws2[BN * kWRow];
+
+  // XCD b % 8 owns the N-tile columns nt = 8 c + xcd.  Its workgroups walk those columns in
+  // groups of group_n: inside a group the M-tiles are walked with the group's columns innermost,
+  // so the ~32 workgroups resident on an XCD form a patch of (32 / group_n) x panels times
+  // group_n W panels and the XCD's L2 fetches each panel once per K-tile.
   const int xcd = blockIdx.x & 7;
   const int local = blockIdx.x >> 3;
-  const int mt = local % p.m_tiles;
-  const int nt = (local / p.m_tiles) * 8 + xcd;
+  const int per_group = p.group_n * p.m_tiles;
+  const int within = local % per_group;
+  const int mt = within / p.group_n;
+  const int nt = ((local / per_group) * p.group_n + within % p.group_n) * 8 + xcd;
   if (nt >= p.n_tiles) return;
   const int n0 = nt * BN, m0 = mt * BM;
   const int split = blockIdx.y;
@@ -363,9 +266,52 @@ void gemm_pipe_kernel(const GemmParams p) {
   const int nkt = (k_end - k_begin) / kBK;
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
+  const unsigned int wave_u = __builtin_amdgcn_readfirstlane(wave);
   const int wn = wave % WAVES_N, wm = wave / WAVES_N;
   const int r = lane & 31, kg = lane >> 5;
   const int64_t ldw_bytes = W8 ? p.K : static_cast<int64_t>(p.K) * 2;
+
+  // copy side: byte offset of this lane's piece for each pass, relative to the tile's first row
+  // (rows past the end are clamped to the last row; their results are never stored)
+  const unsigned char *xbase = p.x + m0 * p.ldx_bytes + static_cast<int64_t>(k_begin) * 2;
+  const unsigned char *wbase = p.w + n0 * ldw_bytes + static_cast<int64_t>(k_begin) * (W8 ? 1 : 2);
+  unsigned int xoff[XP], woff[WP];
+  {
+    const int rl = wave * 8 + (lane >> 3);  // row inside a pass of NW * 8 rows
+    const int piece = (lane & 7) ^ ((rl >> 1) & 7);
+#pragma unroll
+    for (int q = 0; q < XP; ++q) {
+      const int row = min(m0 + q * (NW * 8) + rl, p.M - 1) - m0;
+      xoff[q] = static_cast<unsigned int>(row * p.ldx_bytes + piece * 16);
+    }
+    if constexpr (W8) {
+      const int rw = wave * 16 + (lane >> 2);  // row inside a pass of NW * 16 rows
+      const int pw = (lane & 3) ^ ((rw >> 2) & 3);
+#pragma unroll
+      for (int q = 0; q < WP; ++q) {
+        const int row = min(n0 + q * (NW * 16) + rw, p.N - 1) - n0;
+        woff[q] = static_cast<unsigned int>(row * ldw_bytes + pw * 16);
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < WP; ++q) {
+        const int row = min(n0 + q * (NW * 8) + rl, p.N - 1) - n0;
+        woff[q] = static_cast<unsigned int>(row * ldw_bytes + piece * 16);
+      }
+    }
+  }
+  // fragment side: LDS byte offsets of this lane's pieces
+  const int xrow = (wm * WM + r) * 128;
+  const int wrow = (wn * WN + r) * kWRow;
+  int xq[4], wq[2];
+#pragma unroll
+  for (int s = 0; s < 4; ++s) {
+    // int8 weights: step (ksp, h) = (s>>1, s&1) uses x piece (2*ksp + kg)*2 + h; bf16: piece 2*ks + kg
+    const int c = W8 ? ((s >> 1) * 2 + kg) * 2 + (s & 1) : s * 2 + kg;
+    xq[s] = (c ^ ((r >> 1) & 7)) * 16;
+  }
+#pragma unroll
+  for (int s = 0; s < 2; ++s) wq[s] = ((s * 2 + kg) ^ ((r >> 2) & 3)) * 16;
 
   floatx16 acc[TN][TM];
 #pragma unroll
@@ -375,34 +321,37 @@ void gemm_pipe_kernel(const GemmParams p) {
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  PipeLoader<BN, W8> w0, w1;
-  PipeLoader<BM, false> x0, x1;
-  w0.load(p.w, ldw_bytes, n0, p.N, k_begin, tid);
-  x0.load(p.x, p.ldx_bytes, m0, p.M, k_begin, tid);
-  {
-    const int k1 = k_begin + min(1, nkt - 1) * kBK;
-    w1.load(p.w, ldw_bytes, n0, p.N, k1, tid);
-    x1.load(p.x, p.ldx_bytes, m0, p.M, k1, tid);
+  TLF_DL_ISSUE(Xs0, Ws0, 0)
+  if constexpr (NS == 3) {
+    TLF_DL_ISSUE(Xs1, Ws1, 1)
+    const int triples = nkt / 3;
+    for (int t = 0; t < 3 * triples; t += 3) {
+      TLF_DL_STEP(Xs0, Ws0, Xs2, Ws2, t)
+      TLF_DL_STEP(Xs1, Ws1, Xs0, Ws0, t + 1)
+      TLF_DL_STEP(Xs2, Ws2, Xs1, Ws1, t + 2)
+    }
+    const int rem = nkt - 3 * triples;
+    if (rem >= 1) TLF_DL_STEP(Xs0, Ws0, Xs2, Ws2, 3 * triples)
+    if (rem >= 2) TLF_DL_STEP(Xs1, Ws1, Xs0, Ws0, 3 * triples + 1)
+  } else {
+    const int pairs = nkt / 2;
+    for (int t = 0; t < 2 * pairs; t += 2) {
+      TLF_DL_STEP2(Xs0, Ws0, Xs1, Ws1, t)
+      TLF_DL_STEP2(Xs1, Ws1, Xs0, Ws0, t + 1)
+    }
+    if (nkt & 1) TLF_DL_STEP2(Xs0, Ws0, Xs1, Ws1, nkt - 1)
   }
-  w0.template store_part<0, 1>(Ws[0], tid);
-  x0.template store_part<0, 1>(Xs[0], tid);
-  lds_barrier();
-  // tile t sits in buffer t & 1; set 1 holds tile t+1 at even t, set 0 at odd t
-  const int pairs = nkt / 2;
-  for (int t = 0; t < 2 * pairs; t += 2) {
-    TLF_PIPE_STEP(0, w0, x0, w1, x1, t)
-    TLF_PIPE_STEP(1, w1, x1, w0, x0, t + 1)
-  }
-  if (nkt & 1) {  // the last tile of an odd count sits in buffer 0 (written by the last odd step)
-    TLF_PIPE_MFMA(0, 0)
-    TLF_PIPE_MFMA(0, 1)
-    TLF_PIPE_MFMA(0, 2)
-    TLF_PIPE_MFMA(0, 3)
-  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped copies of the last two steps must land before LDS is released
   gemm_epilogue<TN, TM, WN, WM, W8>(p, acc, m0, n0, wn, wm, r, kg, split);
 }
-#undef TLF_PIPE_STEP
-#undef TLF_PIPE_MFMA
+#undef TLF_DL_STEP
+#undef TLF_DL_STEP2
+#undef TLF_DL_COMPUTE
+#undef TLF_DL_ISSUE
+#undef TLF_DL_ISSUE_PART
+#undef TLF_DL_AFTER_GROUP
+#undef TLF_DL_ISSUE_SETUP
+#undef TLF_DL_COPY
 
 // Sum the split-K partials, apply the channel scale, round once to bf16.
 template <bool W8>
@@ -507,8 +456,8 @@ __global__ __launch_bounds__(512) void skinny_gemm_kernel(const GemmParams p) {
         Pack16 lo, hi;
         if (W8) {
           const uint4 q = wraw[u][t][0];
-          const uint2 c0 = TileLoader<64, true>::cvt4(q.x), c1 = TileLoader<64, true>::cvt4(q.y);
-          const uint2 c2 = TileLoader<64, true>::cvt4(q.z), c3 = TileLoader<64, true>::cvt4(q.w);
+          const uint2 c0 = cvt4_i8_bf16(q.x), c1 = cvt4_i8_bf16(q.y);
+          const uint2 c2 = cvt4_i8_bf16(q.z), c3 = cvt4_i8_bf16(q.w);
           lo.u = make_uint4(c0.x, c0.y, c1.x, c1.y);
           hi.u = make_uint4(c2.x, c2.y, c3.x, c3.y);
         } else {
@@ -598,17 +547,18 @@ int launch_skinny(const GemmParams &p, hipStream_t stream) {
 }
 
 struct GemmPlan {
-  bool pipe = false;  // use the pipelined kernel (tiles up to 128 x 128)
-  int nbuf = 2; // LDS buffers
-  int bn, bm;   // tile
-  int splits;   // split-K factor
+  int bn, bm;         // tile: output channels x tokens
+  int stages;         // LDS stages (2 or 3)
+  int occ;            // waves per SIMD the kernel's registers are budgeted for
+  int splits;         // split-K factor
   int k_per_split;
+  int group_n = 1;    // N-tile columns per XCD patch
 };
 
-// Tile and split-K choice, from a sweep over the Qwen3-8B projection shapes on MI355X.
-// A K-tile step of this kernel costs roughly the same whatever the tile (it is latency bound),
-// so mid-size problems want many small tiles plus a moderate split of K (each split keeps at
-// least 16 K-tiles), and only problems with thousands of tiles use the large MFMA-friendly tiles.
+// Tile, stage and split-K choice, from sweeps over the Qwen3-8B projection shapes on MI355X
+// (M from 24 to 8192, int8 and bf16 weights).  Few tiles: small tiles and a split of K so that
+// about a thousand workgroups exist (each split keeps at least 16 K-tiles); from 256 tiles of
+// 128 x 128 on: no split; from 1024 on: 256 channels x 128 tokens.
 inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
   GemmPlan g;
   auto tiles = [&](int bn, int bm) { return ((N + bn - 1) / bn) * ((M + bm - 1) / bm); };
@@ -617,22 +567,20 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
   const int max_split = ktiles / 16 > 1 ? pow2_floor(ktiles / 16) : 1;
   int splits = 1;
   if (tiles(64, 64) <= 512) {
-    g.bn = 64; g.bm = 64;
+    g.bn = 64; g.bm = 64; g.stages = 2; g.occ = 4;
     splits = pow2_floor(1024 / tiles(64, 64));
-  } else if (tiles(128, 128) <= 1024) {
-    g.bn = 128; g.bm = 128;
-    splits = tiles(128, 128) <= 256 ? pow2_floor(512 / tiles(128, 128)) : 1;
-    // plenty of tiles: one LDS buffer, so that three workgroups share a CU (measured +5-15 %)
-    if (tiles(128, 128) > 256) g.nbuf = 1;
+  } else if (tiles(128, 128) < 256) {
+    g.bn = 128; g.bm = 64; g.stages = 2; g.occ = 3;
+    splits = pow2_floor(1024 / tiles(128, 64));
+  } else if (tiles(128, 128) < 1024) {
+    g.bn = 128; g.bm = 128; g.stages = 3; g.occ = 2;
+  } else if (w8) {
+    g.bn = 256; g.bm = 128; g.stages = 2; g.occ = 2;  // 64 KB of LDS: two workgroups per CU
   } else {
-    // thousands of tiles: 128 channels x 256 tokens, one LDS buffer, two workgroups per CU
-    // (measured 427 us against 456 us for a 256 x 256 tile on 24576 x 4096 at M = 2048)
-    g.bn = 128; g.bm = 256; g.nbuf = 1;
-    // the bf16-weight variant of that tile does not fit 256 registers: keep the 256 x 256 tile
-    if (!w8) { g.bn = 256; g.bm = 256; g.nbuf = 2; }
+    g.bn = 256; g.bm = 128; g.stages = 3; g.occ = 1;
   }
-  // small tiles with two LDS buffers run the pipelined schedule (measured 5-25 % faster)
-  g.pipe = g.bn <= 128 && g.bm <= 128 && g.nbuf == 2;
+  // a long K wants a split of its own: no workgroup walks more than ~48 K-tiles when splitting
+  if (splits > 1 && splits < pow2_floor(ktiles / 48)) splits = pow2_floor(ktiles / 48);
   if (splits > max_split) splits = max_split;
   if (splits > 16) splits = 16;
   if (splits < 1) splits = 1;
@@ -642,20 +590,18 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
   return g;
 }
 
-// TLF_GEMM_PLAN="bn,bm,splits" forces one plan (tuning sweeps); TLF_GEMM_SKINNY_MAX_M moves the
-// hand-over point between the skinny and the tiled kernel.
+// TLF_GEMM_PLAN="bn,bm,splits,stages,occ" forces one plan (tuning sweeps); TLF_GEMM_SKINNY_MAX_M
+// moves the hand-over point between the skinny and the tiled kernel.
 inline bool plan_override(GemmPlan &g, int K) {
   const char *e = getenv("TLF_GEMM_PLAN");
   if (!e) return false;
-  int bn = 0, bm = 0, sp = 0, nb = 2;
-  if (sscanf(e, "%d,%d,%d,%d", &bn, &bm, &sp, &nb) < 3) return false;
-  g.nbuf = nb == 1 ? 1 : 2;
-  g.pipe = nb == 3;
+  int bn = 0, bm = 0, sp = 0, st = 0, occ = 0;
+  if (sscanf(e, "%d,%d,%d,%d,%d", &bn, &bm, &sp, &st, &occ) < 5) return false;
   const int ktiles = K / kBK;
   if (sp < 1) sp = 1;
   if (sp > ktiles) sp = ktiles;
   const int kt_per = (ktiles + sp - 1) / sp;
-  g.bn = bn; g.bm = bm;
+  g.bn = bn; g.bm = bm; g.stages = st; g.occ = occ;
   g.k_per_split = kt_per * kBK;
   g.splits = (ktiles + kt_per - 1) / kt_per;
   return true;
@@ -683,7 +629,7 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   p.partial = nullptr;
   p.M = M; p.N = N; p.K = K;
   if (M <= skinny_max_m()) {
-    p.k_per_split = K; p.splits = 1; p.m_tiles = 1; p.n_tiles = 1;
+    p.k_per_split = K; p.splits = 1; p.m_tiles = 1; p.n_tiles = 1; p.group_n = 1;
     return launch_skinny<W8>(p, stream);
   }
   GemmPlan g = plan_gemm(M, N, K, W8);
@@ -698,38 +644,35 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
       return TLF_E_WORKSPACE;
     p.partial = static_cast<float *>(workspace);
   }
-  const dim3 grid(((p.n_tiles + 7) / 8) * 8 * p.m_tiles, g.splits);
-#define TLF_TILE(BN_, BM_, WN_, WM_)                                                               \
-  if (g.bn == BN_ && g.bm == BM_) {                                                                \
-    if (g.nbuf == 1)                                                                               \
-      hipLaunchKernelGGL((gemm_kernel<BN_, BM_, WN_, WM_, W8, 1>), grid, dim3(256), 0, stream, p); \
-    else                                                                                           \
-      hipLaunchKernelGGL((gemm_kernel<BN_, BM_, WN_, WM_, W8, 2>), grid, dim3(256), 0, stream, p); \
-    launched = true;                                                                               \
+  // XCD patch: group as many N-tile columns as divide this XCD's share evenly (up to 4), once
+  // there are enough M-tiles for the patch to matter
+  {
+    const int cols = (p.n_tiles + 7) / 8;
+    if (p.m_tiles >= 8) g.group_n = cols % 4 == 0 ? 4 : cols % 3 == 0 ? 3 : cols % 2 == 0 ? 2 : 1;
+    if (const char *e = getenv("TLF_GEMM_GROUP_N")) g.group_n = atoi(e) > 0 ? atoi(e) : 1;
   }
+  p.group_n = g.group_n;
+  const int cols_per_xcd = ((p.n_tiles + 7) / 8 + g.group_n - 1) / g.group_n * g.group_n;
+  const dim3 grid(cols_per_xcd * 8 * p.m_tiles, g.splits);
   bool launched = false;
-  if (g.pipe && g.bm <= 128 && g.bn <= 128) {
-#define TLF_PIPE(BN_, BM_, WN_, WM_)                                                                \
-  if (g.bn == BN_ && g.bm == BM_) {                                                                 \
-    hipLaunchKernelGGL((gemm_pipe_kernel<BN_, BM_, WN_, WM_, W8>), grid, dim3(256), 0, stream, p);  \
-    launched = true;                                                                                \
+#define TLF_TILE(BN_, BM_, WN_, WM_, NS_, OCC_)                                             \
+  if (!launched && g.bn == BN_ && g.bm == BM_ && g.stages == NS_ && g.occ == OCC_) {        \
+    hipLaunchKernelGGL((gemm_dlds_kernel<BN_, BM_, WN_, WM_, W8, NS_, OCC_>), grid,         \
+                       dim3(WN_ * WM_ * 64), 0, stream, p);                                 \
+    launched = true;                                                                        \
   }
-    TLF_PIPE(128, 128, 2, 2)
-    TLF_PIPE(64, 128, 1, 4)
-    TLF_PIPE(128, 64, 4, 1)
-    TLF_PIPE(64, 64, 2, 2)
-#undef TLF_PIPE
+  if constexpr (W8) {
+    TLF_TILE(256, 256, 2, 2, 3, 1)  // 144 KB of LDS with int8 weights only
   }
-  if (!launched) {
-  TLF_TILE(256, 256, 2, 2)
-  TLF_TILE(128, 256, 2, 2)
-  TLF_TILE(64, 256, 1, 4)
-  TLF_TILE(256, 128, 2, 2)
-  TLF_TILE(128, 128, 2, 2)
-  TLF_TILE(64, 128, 1, 4)
-  TLF_TILE(128, 64, 4, 1)
-  TLF_TILE(64, 64, 2, 2)
-  }
+  TLF_TILE(256, 128, 2, 2, 3, 1)
+  TLF_TILE(256, 128, 2, 2, 2, 2)
+  TLF_TILE(128, 256, 2, 2, 3, 1)
+  TLF_TILE(128, 256, 2, 2, 2, 2)
+  TLF_TILE(128, 128, 2, 2, 3, 2)
+  TLF_TILE(128, 128, 2, 2, 2, 3)
+  TLF_TILE(128, 64, 4, 1, 2, 3)
+  TLF_TILE(64, 128, 1, 4, 2, 3)
+  TLF_TILE(64, 64, 2, 2, 2, 4)
 #undef TLF_TILE
   if (!launched) return TLF_E_UNSUPPORTED;
   int rc = launch_status();
