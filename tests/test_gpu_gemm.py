@@ -42,6 +42,9 @@ SHAPES = [  # (M, N, K)
     (1, 6144, 4096), (16, 4096, 4096), (64, 1024, 3072), (256, 4096, 4096), (300, 6144, 1024),
     (512, 4096, 1024), (4, 1024, 2048), (2048, 1024, 1024), (257, 24576, 4096), (33, 4096, 12288),
     (128, 5120, 8192), (7, 272, 64),
+    # large-tile plans: ragged M and N with 5 K-tiles, an XCD patch of 4 columns with 3 K-tiles,
+    # and the 128 x 64 tile with a split of K
+    (2050, 8208, 320), (1100, 8192, 192), (512, 6144, 2048), (17, 1040, 64),
 ]
 
 
@@ -79,7 +82,8 @@ def test_w8a16_strided_activations_and_3d_input():
     check(got, exact, exact.to(BF), absdot)
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 4096, 1024), (4, 151936, 1024), (512, 4096, 1024), (256, 6144, 4096), (2048, 3072, 1024), (77, 1024, 3072)])
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 1024), (4, 151936, 1024), (512, 4096, 1024), (256, 6144, 4096), (2048, 3072, 1024), (77, 1024, 3072),
+                                   (2050, 8208, 320), (1100, 8192, 192), (512, 6144, 2048)])
 def test_bf16_gemm(M, N, K):
     from tinyllmforge_amd import ops as P
     x = torch.randn(M, K, generator=g(M)).to(BF)
