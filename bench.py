@@ -55,6 +55,7 @@ def parse():
     ap.add_argument("--num-seqs", type=int, default=256)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--skip-bf16", action="store_true", help="e2e: skip the second run with bf16 linears (profiling)")
     return ap.parse_args()
 
 
@@ -213,7 +214,7 @@ def cpu_baseline_decode(case, budget_s=20.0):
 GEMM_SHAPES = {"qkv": (6144, 4096), "o_proj": (4096, 4096), "gate_up": (24576, 4096), "down": (4096, 12288)}
 
 
-def bench_gemm(args, ms=(1, 16, 64, 256, 2048)):
+def bench_gemm(args, ms=(1, 16, 64, 256, 2048, 8192)):
     import torch
     from tinyllmforge_amd import ops as P
     torch.manual_seed(0)
@@ -262,6 +263,7 @@ def bench_c5(args):
     res = dict(tok_s=round(32 * 256 / wall, 1), wall_s=round(wall, 3), prompt_tokens=sum(len(p) for p in prompts),
                prefill_s=round(st["prefill_time"], 3), decode_s=round(st["decode_time"], 3),
                decode_ms_per_step=round(1e3 * st["decode_time"] / max(1, st["decode_steps"]), 3),
+               prefill_steps=st["prefill_steps"], decode_steps=st["decode_steps"],
                kv_blocks=llm.config.num_kvcache_blocks, kv_dtype="fp8_e4m3")
     llm.exit()
     return res
@@ -366,6 +368,16 @@ def main():
     extra["hbm_probe"] = bench_probes(args)
     if args.workload in ("gemm", "all"):
         extra["w8a16_gemm"] = bench_gemm(args)
+    if args.workload == "gemm":   # its own line: the linear-layer microbench (BASELINE.json configs[2])
+        best = max(r["TFLOPs"] for r in extra["w8a16_gemm"])
+        print(json.dumps({
+            "metric": "W8A16 GEMM TFLOP/s vs bf16 MFMA peak", "value": best, "unit": "TFLOP/s", "n_gpus": 1, "steps": 100,
+            "warmup": 10, "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "BASELINE.json configs[2]: y = x W^T, int8 per-channel weights, bf16 activations, the four "
+                                   "Qwen3-8B projection shapes, M = 1 ... 8192, random normal x, random int8 W"},
+            "roofline": roofline, "cpu_baseline": None, "extra": extra}))
+        return
     if args.workload == "decode_attn":
         cpu = None if args.no_cpu_baseline else cpu_baseline_decode(attn["case"])
         out = {
@@ -381,13 +393,29 @@ def main():
     del attn
     torch.cuda.empty_cache()
     if args.workload in ("c5", "all"):
-        extra["config5_qwen3_32b_fp8kv"] = bench_c5(args)
+        c5 = bench_c5(args)
+        extra["config5_qwen3_32b_fp8kv"] = c5
         import gc
         gc.collect()
         torch.cuda.empty_cache()
+        if args.workload == "c5":   # its own line: same metric on the 32B-shape configuration
+            steps = c5["prefill_steps"] + c5["decode_steps"]
+            print(json.dumps({
+                "metric": "output tok/s (Qwen3-32B-shape, 1 GPU); paged-decode HBM GB/s vs peak", "value": c5["tok_s"],
+                "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": 1,
+                "ms_per_step": round(1e3 * c5["wall_s"] / max(1, steps), 4), "higher_is_better": True,
+                "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                "config": {"workload": "BASELINE.json configs[4]: Qwen3-32B-shaped decoder, random-init, W8A16 linears, "
+                                       "e4m3 KV cache, 32 sequences, prompts ~U[2048,8192] tokens (half share a cached "
+                                       "1024-token prefix), 256 greedy output tokens each, hipGraph decode",
+                           "roofline_workload": "BASELINE.json configs[1] paged decode attention microbench"},
+                "roofline": roofline, "cpu_baseline": None, "extra": extra}))
+            return
     w8, _ = bench_e2e(args, "w8a16")
-    bf, cpu = bench_e2e(args, None)
-    extra["bf16_linears"] = {"tok_s": round(bf["tok_s"], 1), "wall_s": round(bf["wall_s"], 3), "stats": bf["stats"]}
+    cpu = None
+    if not args.skip_bf16:
+        bf, cpu = bench_e2e(args, None)
+        extra["bf16_linears"] = {"tok_s": round(bf["tok_s"], 1), "wall_s": round(bf["wall_s"], 3), "stats": bf["stats"]}
     extra["w8a16_linears"] = {"tok_s": round(w8["tok_s"], 1), "wall_s": round(w8["wall_s"], 3), "stats": w8["stats"],
                               "kv_blocks": w8["kv_blocks"]}
     steps = w8["stats"]["steps"]
