@@ -60,7 +60,7 @@ def parse():
 
 
 # ----------------------------------------------------------------------------- config 2
-def make_decode_case(batch=64, hq=32, hkv=8, dh=128, bs=256, pool=2048, seed=0, device="cuda"):
+def make_decode_case(batch=64, hq=32, hkv=8, dh=128, bs=256, pool=2048, seed=0, device="cuda", fp8=False):
     import torch
     from tinyllmforge_amd import ops as P
     g = torch.Generator().manual_seed(seed)
@@ -80,20 +80,22 @@ def make_decode_case(batch=64, hq=32, hkv=8, dh=128, bs=256, pool=2048, seed=0, 
     total = int(ctx.sum())
     dev = torch.device(device)
     torch.manual_seed(seed)
-    k_cache = torch.zeros(pool, bs, hkv, dh, dtype=torch.bfloat16, device=dev)
-    v_cache = torch.zeros(pool, bs, hkv, dh, dtype=torch.bfloat16, device=dev)
+    cache_dtype = torch.float8_e4m3fn if fp8 else torch.bfloat16
+    k_cache = torch.zeros(pool, bs, hkv, dh, dtype=cache_dtype, device=dev)
+    v_cache = torch.zeros(pool, bs, hkv, dh, dtype=cache_dtype, device=dev)
+    scales = dict(k_scale=torch.full((hkv,), 0.02, device=dev), v_scale=torch.full((hkv,), 0.02, device=dev)) if fp8 else {}
     slots_d = slots.to(dev)
     chunk = 32768
     for s in range(0, total, chunk):                       # K/V rows go in through the store kernel
         n = min(chunk, total - s)
         kv = torch.randn(n, 2 * hkv * dh, device=dev, dtype=torch.float32).to(torch.bfloat16)
         P.store_kvcache(kv[:, :hkv * dh].view(n, hkv, dh), kv[:, hkv * dh:].view(n, hkv, dh),
-                        k_cache, v_cache, slots_d[s:s + n])
+                        k_cache, v_cache, slots_d[s:s + n], **scales)
     q = torch.randn(batch, hq, dh, device=dev, dtype=torch.float32).to(torch.bfloat16)
-    algo_bytes = total * hkv * dh * 2 * 2 + 2 * batch * hq * dh * 2 + batch * (maxb + 1) * 4
+    algo_bytes = total * hkv * dh * 2 * (1 if fp8 else 2) + 2 * batch * hq * dh * 2 + batch * (maxb + 1) * 4
     return dict(q=q, k_cache=k_cache, v_cache=v_cache, ctx=ctx.to(torch.int32).to(dev), bt=bt.to(dev),
                 scale=1.0 / math.sqrt(dh), algo_bytes=algo_bytes, total_tokens=total,
-                ctx_cpu=ctx, bt_cpu=bt)
+                ctx_cpu=ctx, bt_cpu=bt, scales=scales)
 
 
 def time_launches(fn, steps, warmup):
@@ -159,14 +161,14 @@ def bench_probes(args):
                 copy_GBps=round(2 * n / (tc["mean_ms"] * 1e-3) / 1e9, 1), bytes=n)
 
 
-def bench_decode_attn(args):
+def bench_decode_attn(args, fp8=False, hq=32):
     import torch
     from tinyllmforge_amd import ops as P
-    case = make_decode_case(batch=args.batch)
+    case = make_decode_case(batch=args.batch, fp8=fp8, hq=hq)
 
     def step():
         return P.paged_decode_attention(case["q"], case["k_cache"], case["v_cache"], case["ctx"], case["bt"],
-                                        case["scale"])
+                                        case["scale"], **case["scales"])
 
     t = time_launches(step, args.attn_steps, 30)
     # "step" time = back-to-back launches over the timed region (what a decode loop sees)
@@ -176,8 +178,8 @@ def bench_decode_attn(args):
     res = dict(ms_per_step=ms_per_step, value=gbps,
                roofline=dict(bound="hbm", achieved=round(kern_gbps, 1), peak=HBM_PEAK_GBPS, unit="GB/s",
                              frac=round(kern_gbps / HBM_PEAK_GBPS, 4),
-                             traffic=DECODE_ATTN_TRAFFIC_BYTES if args.batch == 64 else None,
-                             kernel="paged_decode_kernel<8,false> + paged_decode_merge_kernel",
+                             traffic=DECODE_ATTN_TRAFFIC_BYTES if args.batch == 64 and not fp8 and hq == 32 else None,
+                             kernel="paged_decode_kernel<8,%s> + paged_decode_merge_kernel" % ("true" if fp8 else "false"),
                              launch_ms_mean=round(t["mean_ms"], 5), launch_ms_median=round(t["median_ms"], 5),
                              launch_ms_min=round(t["min_ms"], 5), algorithmic_bytes=case["algo_bytes"]),
                case=case)
@@ -264,6 +266,8 @@ def bench_c5(args):
                prefill_s=round(st["prefill_time"], 3), decode_s=round(st["decode_time"], 3),
                decode_ms_per_step=round(1e3 * st["decode_time"] / max(1, st["decode_steps"]), 3),
                prefill_steps=st["prefill_steps"], decode_steps=st["decode_steps"],
+               cached_prompt_tokens=st["cached_prompt_tokens"],
+               decode_byte_floor=decode_byte_floor(llm.config.hf_config, st, "w8a16", kv_itemsize=1),
                kv_blocks=llm.config.num_kvcache_blocks, kv_dtype="fp8_e4m3")
     llm.exit()
     return res
@@ -318,7 +322,8 @@ def bench_e2e(args, quantization):
                      decode_steps=st["decode_steps"], prefill_s=round(st["prefill_time"], 3),
                      decode_s=round(st["decode_time"], 3),
                      decode_ms_per_step=round(1e3 * st["decode_time"] / max(1, st["decode_steps"]), 3))
-    model_params = {k: v.data for k, v in llm.model_runner.model.named_parameters()} if quantization is None else None
+    if "decode_context_tokens" in (llm.last_stats or {}) and args.steps == 0:
+        stats["decode_byte_floor"] = decode_byte_floor(llm.config.hf_config, llm.last_stats, quantization, kv_itemsize=2)
     res = dict(tok_s=total / wall, wall_s=wall, total_output_tokens=total, init_s=round(init_s, 1), stats=stats,
                kv_blocks=llm.config.num_kvcache_blocks)
     cpu = None
@@ -330,6 +335,20 @@ def bench_e2e(args, quantization):
     gc.collect()
     torch.cuda.empty_cache()
     return res, cpu
+
+
+def decode_byte_floor(hf, st, quantization, kv_itemsize):
+    """Bytes a decode phase cannot avoid: every linear weight (and the bf16 LM head) once per step plus every
+    context token's K and V row once per layer; the time they take at the HBM peak, beside the measured time."""
+    h, i, L = hf.hidden_size, hf.intermediate_size, hf.num_hidden_layers
+    hq, hkv, dh, v = hf.num_attention_heads, hf.num_key_value_heads, hf.head_dim, hf.vocab_size
+    lin = L * ((hq + 2 * hkv) * dh * h + hq * dh * h + 2 * i * h + h * i)
+    w_step = lin * (1 if quantization == "w8a16" else 2) + v * h * 2
+    kv = st["decode_context_tokens"] * hkv * dh * 2 * kv_itemsize * L
+    floor_s = (st["decode_steps"] * w_step + kv) / (HBM_PEAK_GBPS * 1e9)
+    return dict(weight_GB_per_step=round(w_step / 1e9, 3), kv_GB_total=round(kv / 1e9, 1),
+                floor_s_at_hbm_peak=round(floor_s, 3), measured_s=round(st["decode_time"], 3),
+                frac=round(floor_s / max(st["decode_time"], 1e-9), 4))
 
 
 def cpu_baseline_e2e(llm, prompts, nseq=2, out_tokens=4):
@@ -393,7 +412,11 @@ def main():
     del attn
     torch.cuda.empty_cache()
     if args.workload in ("c5", "all"):
+        a8 = bench_decode_attn(args, fp8=True, hq=64)   # the decode microbench on e4m3 rows, 64 query heads
+        a8.pop("case")
+        torch.cuda.empty_cache()
         c5 = bench_c5(args)
+        c5["paged_decode_fp8_rows"] = a8["roofline"]
         extra["config5_qwen3_32b_fp8kv"] = c5
         import gc
         gc.collect()

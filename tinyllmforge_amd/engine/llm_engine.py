@@ -52,6 +52,10 @@ class LLMEngine:
         self.scheduler.postprocess(seqs, token_ids)
         outputs = [(s.seq_id, s.completion_token_ids) for s in seqs if s.is_finished]
         num_tokens = sum(len(s) for s in seqs) if is_prefill else -len(seqs)
+        # for the statistics of generate(): cached prompt tokens of a prefill step, context tokens a
+        # decode step's attention reads (the token stored in this step included)
+        self._step_info = (sum(s.num_cached_tokens for s in seqs) if is_prefill else 0,
+                           0 if is_prefill else sum(len(s) - 1 for s in seqs))
         return outputs, num_tokens
 
     def is_finished(self):
@@ -64,7 +68,7 @@ class LLMEngine:
             self.add_request(prompt, sp)
         done = {}
         stats = dict(prefill_steps=0, decode_steps=0, prefill_tokens=0, decode_tokens=0,
-                     prefill_time=0.0, decode_time=0.0)
+                     prefill_time=0.0, decode_time=0.0, cached_prompt_tokens=0, decode_context_tokens=0)
         while not self.is_finished():
             t0 = perf_counter()
             finished, num_tokens = self.step()
@@ -73,6 +77,8 @@ class LLMEngine:
             stats[f"{kind}_steps"] += 1
             stats[f"{kind}_tokens"] += abs(num_tokens)
             stats[f"{kind}_time"] += dt
+            stats["cached_prompt_tokens"] += self._step_info[0]
+            stats["decode_context_tokens"] += self._step_info[1]
             for seq_id, toks in finished:
                 done[seq_id] = toks
         self.last_stats = stats
