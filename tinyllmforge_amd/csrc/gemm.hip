@@ -153,14 +153,16 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
 // Copy slices issued after MFMA group G (0..3) of a step.  Three stages: one slice per group.
 // Two stages: the copy has to land within the step, so everything goes out in its first half.
 #define TLF_DL_AFTER_GROUP(G)                          \
-  if constexpr (NS == 3) {                             \
-    if ((G) == 0) TLF_DL_ISSUE_PART(0)                 \
-    if ((G) == 1) TLF_DL_ISSUE_PART(1)                 \
-    if ((G) == 2) TLF_DL_ISSUE_PART(2)                 \
-    if ((G) == 3) TLF_DL_ISSUE_PART(3)                 \
-  } else {                                             \
-    if ((G) == 0) { TLF_DL_ISSUE_PART(0) TLF_DL_ISSUE_PART(1) } \
-    if ((G) == 1) { TLF_DL_ISSUE_PART(2) TLF_DL_ISSUE_PART(3) } \
+  if (do_issue_) {                                     \
+    if constexpr (NS >= 3) {                           \
+      if ((G) == 0) TLF_DL_ISSUE_PART(0)               \
+      if ((G) == 1) TLF_DL_ISSUE_PART(1)               \
+      if ((G) == 2) TLF_DL_ISSUE_PART(2)               \
+      if ((G) == 3) TLF_DL_ISSUE_PART(3)               \
+    } else {                                           \
+      if ((G) == 0) { TLF_DL_ISSUE_PART(0) TLF_DL_ISSUE_PART(1) } \
+      if ((G) == 1) { TLF_DL_ISSUE_PART(2) TLF_DL_ISSUE_PART(3) } \
+    }                                                  \
   }
 // Compute on stage (XS, WS); the four copy slices of the step go between its MFMA groups.
 #define TLF_DL_COMPUTE(XS, WS)                                                                    \
@@ -217,6 +219,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
   {                                                \
     TLF_DL_BARRIER(kLoads);                        \
     TLF_DL_ISSUE_SETUP(XS_NEXT2, WS_NEXT2, (T) + 2) \
+    constexpr bool do_issue_ = true;               \
     TLF_DL_COMPUTE(XS, WS)                         \
   }
 // Two-stage form: the copy of tile T+1 is issued right after the barrier of step T into the stage
@@ -226,6 +229,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
   {                                               \
     TLF_DL_BARRIER(0);                            \
     TLF_DL_ISSUE_SETUP(XS_NEXT, WS_NEXT, (T) + 1) \
+    constexpr bool do_issue_ = true;              \
     TLF_DL_COMPUTE(XS, WS)                        \
   }
 
@@ -237,7 +241,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
 template <int BN, int BM, int WAVES_N, int WAVES_M, bool W8, int NS, int OCC, int KG>
 __global__ __launch_bounds__(WAVES_N * WAVES_M * KG * 64) __attribute__((amdgpu_waves_per_eu(OCC, 8)))
 void gemm_dlds_kernel(const GemmParams p) {
-  static_assert(NS == 2 || NS == 3, "2 or 3 stages");
+  static_assert(NS >= 2 && NS <= 8, "2 to 8 stages");
   constexpr int NW = WAVES_N * WAVES_M;       // waves of one set
   static_assert(NW == 4 || NW == 8, "4 or 8 waves");  // 8: two waves share each SIMD (not faster in the sweeps)
   static_assert(NW * KG <= 16, "at most 1024 threads");
@@ -254,9 +258,9 @@ void gemm_dlds_kernel(const GemmParams p) {
   constexpr int kPool = NS * kStage > kReduce ? NS * kStage : kReduce;
   static_assert(XP >= 1 && WP >= 1 && TN >= 1 && TM >= 1, "tile too small");
   static_assert(kPool <= 160 * 1024, "the stages must fit LDS");
-  static_assert(kLoads <= 31, "vmcnt range");
+  static_assert((NS - 2) * kLoads <= 63, "vmcnt range");
   __shared__ __attribute__((aligned(1024))) unsigned char pool[kPool];
-  unsigned char *const Xs0 = pool, *const Xs1 = pool + kStage, *const Xs2 = pool + (NS - 1) * kStage;
+  unsigned char *const Xs0 = pool, *const Xs1 = pool + kStage, *const Xs2 = pool + 2 * (NS > 2) * kStage;
   unsigned char *const Ws0 = Xs0 + KG * kXBytes, *const Ws1 = Xs1 + KG * kXBytes,
                       *const Ws2 = Xs2 + KG * kXBytes;
 
@@ -348,13 +352,29 @@ void gemm_dlds_kernel(const GemmParams p) {
     const int rem = nkt - 3 * triples;
     if (rem >= 1) TLF_DL_STEP(Xs0, Ws0, Xs2, Ws2, 3 * triples)
     if (rem >= 2) TLF_DL_STEP(Xs1, Ws1, Xs0, Ws0, 3 * triples + 1)
-  } else {
+  } else if constexpr (NS == 2) {
     const int pairs = nkt / 2;
     for (int t = 0; t < 2 * pairs; t += 2) {
       TLF_DL_STEP2(Xs0, Ws0, Xs1, Ws1, t)
       TLF_DL_STEP2(Xs1, Ws1, Xs0, Ws0, t + 1)
     }
     if (nkt & 1) TLF_DL_STEP2(Xs0, Ws0, Xs1, Ws1, nkt - 1)
+  } else {
+    // NS >= 4: a ring of stages addressed at run time, NS-1 tiles in flight.  For shapes whose
+    // workgroups are few and stream from HBM: a CU's copy rate is (bytes in flight) / latency.
+    // Tiles past the end are not requested; the last NS-1 steps then wait for everything.
+    for (int t = 1; t < NS - 1; ++t)
+      if (t < nkt) TLF_DL_ISSUE(pool + t * kStage, pool + t * kStage + KG * kXBytes, t)
+    int cur = 0;
+    for (int t = 0; t < nkt; ++t) {
+      const int nxt = cur == 0 ? NS - 1 : cur - 1;  // the stage tile t-1 was read from
+      unsigned char *const xs = pool + cur * kStage, *const xn = pool + nxt * kStage;
+      const bool do_issue_ = t + NS - 1 < nkt;
+      if (do_issue_) TLF_DL_BARRIER((NS - 2) * kLoads); else TLF_DL_BARRIER(0);
+      TLF_DL_ISSUE_SETUP(xn, xn + KG * kXBytes, t + NS - 1)
+      TLF_DL_COMPUTE(xs, xs + KG * kXBytes)
+      cur = cur + 1 == NS ? 0 : cur + 1;
+    }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the clamped copies of the last two steps must land before LDS is released
   if constexpr (KG > 1) {
@@ -617,6 +637,14 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
       // global memory, no reduce kernel); measured 5-20 % faster on 4096 x 4096 and 6144 x 4096
       g.kgroups = tiles(64, 64) <= 256 ? 4 : 2;
       splits = tiles(64, 64) <= 128 ? 2 : 1;
+      // weights stream from HBM: a third stage keeps two tiles per wave set in flight
+      // (int8 only: 144 KB of LDS; measured 17.1 -> 14.1 us on 4096 x 4096 at M = 130)
+      if (w8 && g.kgroups == 4) g.stages = 3;
+    } else if (M > 64 && ktiles > 64) {
+      // long K (down projection): 128 channels x 64 tokens, split of K, four-stage ring
+      // (measured 42.6 -> 38.2 us at M = 130, 55.7 -> 44.5 us at M = 256 on 4096 x 12288)
+      g.bn = 128; g.bm = 64; g.stages = 4; g.occ = 3;
+      splits = 4;
     }
   } else if (tiles(128, 128) < 256) {
     g.bn = 128; g.bm = 64; g.stages = 2; g.occ = 3;
@@ -738,10 +766,20 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   TLF_TILE(64, 128, 1, 4, 2, 3)
   TLF_TILE(64, 64, 2, 2, 2, 4)
   TLF_TILE_KG(64, 64, 2, 2, 2, 4, 2)
+  TLF_TILE(64, 64, 2, 2, 4, 4)
+  TLF_TILE(64, 64, 2, 2, 8, 4)
+  TLF_TILE_KG(64, 64, 2, 2, 4, 4, 2)
+  TLF_TILE(128, 64, 4, 1, 4, 3)
+  TLF_TILE(128, 64, 4, 1, 6, 3)
+  TLF_TILE(256, 64, 4, 1, 4, 3)
   TLF_TILE_KG(64, 64, 2, 2, 2, 4, 4)
   TLF_TILE_KG(128, 64, 4, 1, 2, 4, 2)
   if constexpr (W8) {
-    TLF_TILE_KG(128, 64, 4, 1, 2, 4, 4)  // 128 KB of LDS with int8 weights only
+    TLF_TILE_KG(128, 64, 4, 1, 2, 4, 4)  // these fit LDS with int8 weights only
+    TLF_TILE_KG(64, 64, 2, 2, 6, 4, 2)
+    TLF_TILE_KG(64, 64, 2, 2, 3, 4, 4)
+    TLF_TILE_KG(128, 64, 4, 1, 4, 4, 2)
+    TLF_TILE(256, 64, 4, 1, 6, 3)
   }
   TLF_TILE_KG(128, 128, 2, 2, 2, 2, 2)
   TLF_TILE(256, 64, 4, 1, 2, 3)
