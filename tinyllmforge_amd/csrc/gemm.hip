@@ -753,38 +753,23 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
     launched = true;                                                                        \
   }
 #define TLF_TILE(BN_, BM_, WN_, WM_, NS_, OCC_) TLF_TILE_KG(BN_, BM_, WN_, WM_, NS_, OCC_, 1)
-  if constexpr (W8) {
-    TLF_TILE(256, 256, 2, 2, 3, 1)  // 144 KB of LDS with int8 weights only
-  }
-  TLF_TILE(256, 128, 2, 2, 3, 1)
-  TLF_TILE(256, 128, 2, 2, 2, 2)
-  TLF_TILE(128, 256, 2, 2, 3, 1)
-  TLF_TILE(128, 256, 2, 2, 2, 2)
-  TLF_TILE(128, 128, 2, 2, 3, 2)
-  TLF_TILE(128, 128, 2, 2, 2, 3)
-  TLF_TILE(128, 64, 4, 1, 2, 3)
-  TLF_TILE(64, 128, 1, 4, 2, 3)
+  // the instances plan_gemm() uses ...
   TLF_TILE(64, 64, 2, 2, 2, 4)
   TLF_TILE_KG(64, 64, 2, 2, 2, 4, 2)
-  TLF_TILE(64, 64, 2, 2, 4, 4)
-  TLF_TILE(64, 64, 2, 2, 8, 4)
-  TLF_TILE_KG(64, 64, 2, 2, 4, 4, 2)
-  TLF_TILE(128, 64, 4, 1, 4, 3)
-  TLF_TILE(128, 64, 4, 1, 6, 3)
-  TLF_TILE(256, 64, 4, 1, 4, 3)
   TLF_TILE_KG(64, 64, 2, 2, 2, 4, 4)
-  TLF_TILE_KG(128, 64, 4, 1, 2, 4, 2)
-  if constexpr (W8) {
-    TLF_TILE_KG(128, 64, 4, 1, 2, 4, 4)  // these fit LDS with int8 weights only
-    TLF_TILE_KG(64, 64, 2, 2, 6, 4, 2)
+  TLF_TILE(128, 64, 4, 1, 2, 3)
+  TLF_TILE(128, 64, 4, 1, 4, 3)
+  TLF_TILE(128, 128, 2, 2, 3, 2)
+  TLF_TILE(256, 128, 2, 2, 2, 2)
+  TLF_TILE(256, 128, 2, 2, 3, 1)
+  if constexpr (W8) {  // these fit LDS with int8 weights only
     TLF_TILE_KG(64, 64, 2, 2, 3, 4, 4)
-    TLF_TILE_KG(128, 64, 4, 1, 4, 4, 2)
-    TLF_TILE(256, 64, 4, 1, 6, 3)
+    TLF_TILE(256, 256, 2, 2, 3, 1)
   }
-  TLF_TILE_KG(128, 128, 2, 2, 2, 2, 2)
+  // ... and alternatives kept for tuning through TLF_GEMM_PLAN
+  TLF_TILE(128, 256, 2, 2, 2, 2)
+  TLF_TILE(128, 128, 2, 2, 2, 3)
   TLF_TILE(256, 64, 4, 1, 2, 3)
-  TLF_TILE_KG(256, 64, 4, 1, 2, 4, 2)
-  TLF_TILE(256, 64, 4, 1, 3, 3)
 #undef TLF_TILE
 #undef TLF_TILE_KG
   if (!launched) return TLF_E_UNSUPPORTED;
