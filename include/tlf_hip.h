@@ -192,6 +192,13 @@ int tlf_bf16_gemm(const void *x, int64_t x_stride, const void *w, void *y,
                   int32_t M, int32_t N, int32_t K,
                   void *workspace, size_t workspace_bytes, void *stream);
 
+/* Diagnostic, no counterpart in the reference, touches no GPU: the kernel plan the two GEMM entry
+ * points would use for a shape.  plan8 = {tile channels, tile tokens, LDS stages, waves/SIMD budget,
+ * K-groups per workgroup, split-K factor, K per split, N-tile columns per XCD patch}; tile 0 x 0
+ * means the skinny kernel.  Returns TLF_OK when a kernel instance exists for the plan,
+ * TLF_E_UNSUPPORTED otherwise (the GEMM call would return the same). */
+int tlf_gemm_plan(int32_t M, int32_t N, int32_t K, int32_t w8, int32_t *plan8);
+
 /* ---------------------------------------------------------------------------
  * a3  paged decode attention   replaces the decode branch layers/attention.py:106-109
  *     (flash_attn_with_kvcache, one query token per sequence)

@@ -58,3 +58,34 @@ def test_ops_refuse_cpu_tensors():
     from tinyllmforge_amd import ops, _lib
     with pytest.raises(_lib.TlfError):
         ops.silu_and_mul(torch.zeros(2, 16, dtype=torch.bfloat16))
+
+
+def test_gemm_plan_has_a_kernel_for_every_shape_the_models_use():
+    """Host-only sweep of the GEMM planner (no GPU call): every token count from 1 to 600 and a few large
+    ones, every projection of the three Qwen3 shapes plus the LM head, int8 and bf16 weights, must map to
+    an existing kernel instance with a consistent split of K that the workspace query covers."""
+    import ctypes
+    from tinyllmforge_amd import _lib
+    lib = _lib.load()
+    shapes = set()
+    for h, hq, hkv, inter in [(1024, 16, 8, 3072), (4096, 32, 8, 12288), (5120, 64, 8, 25600)]:
+        shapes |= {((hq + 2 * hkv) * 128, h), (h, hq * 128), (2 * inter, h), (h, inter), (151936, h)}
+    ms = list(range(1, 601)) + [777, 1024, 2047, 4096, 8192, 16384]
+    plan = (ctypes.c_int32 * 8)()
+    seen = set()
+    for n, k in sorted(shapes):
+        for w8 in (0, 1):
+            for m in ms:
+                rc = lib.tlf_gemm_plan(m, n, k, w8, plan)
+                assert rc == 0, f"no kernel for M={m} N={n} K={k} w8={w8}: rc={rc} plan={list(plan)}"
+                bn, bm, stages, occ, kgroups, splits, k_per_split, group_n = list(plan)
+                seen.add((bn, bm, stages, occ, kgroups))
+                assert k_per_split % 64 == 0 and splits >= 1 and splits * k_per_split >= k
+                assert (splits - 1) * k_per_split < k, "an empty split"
+                if bn:   # tiled kernel
+                    assert (k_per_split // 64) % kgroups == 0 and ((k - (splits - 1) * k_per_split) // 64) % kgroups == 0
+                    assert 1 <= group_n <= 4
+                    if splits > 1:
+                        assert lib.tlf_w8a16_gemm_workspace_bytes(m, n, k) >= splits * m * n * 4
+    assert len(seen) >= 6, seen          # the sweep reaches the skinny kernel and several tile shapes
+    assert lib.tlf_gemm_plan(4, 1024, 100, 1, plan) == -2   # K not a multiple of 64

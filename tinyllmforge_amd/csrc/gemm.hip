@@ -697,10 +697,13 @@ inline int skinny_max_m() {
   return v;
 }
 
+// plan_out != nullptr: nothing is launched; the eight plan fields are written there instead and the
+// return code says whether a kernel instance exists for the plan.
 template <bool W8>
 int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *scale, void *y,
                 int32_t M, int32_t N, int32_t K, void *workspace, size_t workspace_bytes,
-                hipStream_t stream) {
+                hipStream_t stream, int32_t *plan_out = nullptr) {
+  const bool dry = plan_out != nullptr;
   GemmParams p;
   p.x = static_cast<const unsigned char *>(x);
   p.ldx_bytes = x_stride * 2;
@@ -711,6 +714,11 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   p.M = M; p.N = N; p.K = K;
   if (M <= skinny_max_m()) {
     p.k_per_split = K; p.splits = 1; p.m_tiles = 1; p.n_tiles = 1; p.group_n = 1;
+    if (dry) {
+      const int32_t skinny[8] = {0, 0, 0, 0, 1, 1, K, 1};  // tile 0 x 0 = the skinny kernel
+      for (int i = 0; i < 8; ++i) plan_out[i] = skinny[i];
+      return TLF_OK;
+    }
     return launch_skinny<W8>(p, stream);
   }
   GemmPlan g = plan_gemm(M, N, K, W8);
@@ -728,7 +736,7 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   p.splits = g.splits;
   p.m_tiles = (M + g.bm - 1) / g.bm;
   p.n_tiles = (N + g.bn - 1) / g.bn;
-  if (g.splits > 1) {
+  if (g.splits > 1 && !dry) {
     const size_t need = static_cast<size_t>(g.splits) * M * N * sizeof(float);
     if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15u))
       return TLF_E_WORKSPACE;
@@ -748,8 +756,9 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
 #define TLF_TILE_KG(BN_, BM_, WN_, WM_, NS_, OCC_, KG_)                                     \
   if (!launched && g.bn == BN_ && g.bm == BM_ && g.stages == NS_ && g.occ == OCC_ &&        \
       g.kgroups == KG_) {                                                                   \
-    hipLaunchKernelGGL((gemm_dlds_kernel<BN_, BM_, WN_, WM_, W8, NS_, OCC_, KG_>), grid,    \
-                       dim3(WN_ * WM_ * KG_ * 64), 0, stream, p);                           \
+    if (!dry)                                                                               \
+      hipLaunchKernelGGL((gemm_dlds_kernel<BN_, BM_, WN_, WM_, W8, NS_, OCC_, KG_>), grid,  \
+                         dim3(WN_ * WM_ * KG_ * 64), 0, stream, p);                         \
     launched = true;                                                                        \
   }
 #define TLF_TILE(BN_, BM_, WN_, WM_, NS_, OCC_) TLF_TILE_KG(BN_, BM_, WN_, WM_, NS_, OCC_, 1)
@@ -772,6 +781,11 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   TLF_TILE(256, 64, 4, 1, 2, 3)
 #undef TLF_TILE
 #undef TLF_TILE_KG
+  if (dry) {
+    const int32_t fields[8] = {g.bn, g.bm, g.stages, g.occ, g.kgroups, g.splits, g.k_per_split, g.group_n};
+    for (int i = 0; i < 8; ++i) plan_out[i] = fields[i];
+    return launched ? TLF_OK : TLF_E_UNSUPPORTED;
+  }
   if (!launched) return TLF_E_UNSUPPORTED;
   int rc = launch_status();
   if (rc != TLF_OK) return rc;
@@ -823,4 +837,11 @@ extern "C" int tlf_bf16_gemm(const void *x, int64_t x_stride, const void *w, voi
   if (rc != TLF_OK) return rc;
   return launch_gemm<false>(x, x_stride, w, nullptr, y, M, N, K, workspace, workspace_bytes,
                             static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tlf_gemm_plan(int32_t M, int32_t N, int32_t K, int32_t w8, int32_t *plan8) {
+  if (!plan8) return TLF_E_NULL;
+  if (M <= 0 || N <= 0 || K <= 0 || K % kBK || N % 16) return TLF_E_SHAPE;
+  return w8 ? launch_gemm<true>(nullptr, K, nullptr, nullptr, nullptr, M, N, K, nullptr, 0, nullptr, plan8)
+            : launch_gemm<false>(nullptr, K, nullptr, nullptr, nullptr, M, N, K, nullptr, 0, nullptr, plan8);
 }
