@@ -67,7 +67,8 @@ __device__ __forceinline__ void fp8x16_to_bf16(const uint4 &in, uint4 &lo, uint4
 }
 
 template <int CT, bool KV8>
-__global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))  // 256 registers: two workgroups per CU
+void prefill_attn_kernel(const PrefillParams p) {
   __shared__ __attribute__((aligned(16))) unsigned short Ks[kBKV][kPRow];
   __shared__ __attribute__((aligned(16))) unsigned short Vs[kBKV][kPRow];
   const int seq = blockIdx.z;
@@ -207,32 +208,44 @@ __global__ __launch_bounds__(256) void prefill_attn_kernel(const PrefillParams p
       bf16x8 ph[CT], pl[CT];
 #pragma unroll
       for (int c = 0; c < CT; ++c) {
+        // (the softmax is where this kernel's vector-ALU time goes: raw v_exp_f32, one fused
+        // multiply-add per score, no mask arithmetic on tiles that lie wholly below the diagonal)
         float sv[8];
-        const int tbase = kv0 + hh * 32 + g * 8;
-        const int limit = min(shift + urow[c], lk - 1);  // last visible key of this unit
         float mt = -INFINITY;
+        if (need_mask) {  // workgroup-uniform
+          const int tbase = kv0 + hh * 32 + g * 8;
+          const int limit = min(shift + urow[c], lk - 1);  // last visible key of this unit
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          const float raw = (j < 4 ? s0[c][j] : s1[c][j - 4]) * scale_log2;
-          sv[j] = (!need_mask || tbase + j <= limit) ? raw : -INFINITY;
-          mt = fmaxf(mt, sv[j]);
+          for (int j = 0; j < 8; ++j) {
+            const float raw = j < 4 ? s0[c][j] : s1[c][j - 4];
+            sv[j] = tbase + j <= limit ? raw : -INFINITY;
+            mt = fmaxf(mt, sv[j]);
+          }
+        } else {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) {
+            sv[j] = j < 4 ? s0[c][j] : s1[c][j - 4];
+            mt = fmaxf(mt, sv[j]);
+          }
         }
         mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
         mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-        const float m_new = fmaxf(m_run[c], mt);
+        // running max in the scaled (log2) domain; scale_log2 > 0, so scaling commutes with max
+        const float m_new = fmaxf(m_run[c], mt * scale_log2);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = exp2f(m_run[c] - m_use);
+        const float alpha = __builtin_amdgcn_exp2f(m_run[c] - m_use);
         float psum = 0.f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-          const float pv = exp2f(sv[j] - m_use);
+          // p = 2^(s * scale - m): arguments are <= 0, a flushed denormal result is an exact 0 weight
+          const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[j], scale_log2, -m_use));
           psum += pv;
           ph[c][j] = static_cast<__bf16>(pv);
           pl[c][j] = static_cast<__bf16>(pv - static_cast<float>(ph[c][j]));
         }
         l_run[c] = l_run[c] * alpha + psum;
         m_run[c] = m_new;
-        if (alpha != 1.0f) {
+        if (__any(alpha != 1.0f)) {  // wave-uniform: the running max rarely moves after the first tiles
 #pragma unroll
           for (int d = 0; d < 8; ++d)
 #pragma unroll
