@@ -206,55 +206,42 @@ void paged_decode_kernel(const DecodeParams p) {
 
     // Issue the loads of the tile starting at token t0 (a tile never straddles a block);
     // blk is its block-table entry, fetched one tile earlier so that its latency is hidden.
-    // The loads are unconditional, so that the compiler can count them and wait for the oldest
-    // tile only (a conditional load makes it drain the whole queue): tokens past the end re-read
-    // the segment's last row (their scores are masked and their probability is 0), a tile of an
-    // unmapped block reads block 0 and is zeroed before use, and a prefetch past the segment
-    // (real == false) reads one 16-byte piece of a valid row with every lane.
-    auto load_tile = [&](int t0, int64_t blk, bool real, TileRegs<KV8> &r) __attribute__((always_inline)) {
-      const int tc = real ? t0 : t_begin;
-      const int bi = tc / p.block_size;
+    auto load_tile = [&](int t0, int64_t blk, TileRegs<KV8> &r) {
+      const int bi = t0 / p.block_size;
       const bool ok = blk >= 0 && blk < p.num_cache_blocks;
-      const int64_t tok0 = (ok ? blk : 0) * p.block_size - bi * p.block_size;
+      const int64_t tok0 = (ok ? blk : 0) * p.block_size + (t0 - bi * p.block_size);
       r.ok = ok;
 #pragma unroll
       for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
         // bf16: 4 tokens x 16 chunks of 8 elements per instruction; e4m3: 8 tokens x 8 chunks of 16
         const int tt = KV8 ? i * 8 + (lane >> 3) : i * 4 + g;
-        const int tok = real ? min(tc + tt, t_end - 1) : tc;
-        const int piece = real ? (KV8 ? (lane & 7) * 16 : n * 8) : 0;
-        const int64_t off = KV8 ? (tok0 + tok) * row_elems + w * kDh + piece
-                                : ((tok0 + tok) * row_elems + w * kDh + piece) * 2;
-        r.k[i] = load_nt_u4(p.k_cache + off);
-        r.v[i] = load_nt_u4(p.v_cache + off);
+        const int64_t off = KV8 ? (tok0 + tt) * row_elems + w * kDh + (lane & 7) * 16
+                                : ((tok0 + tt) * row_elems + w * kDh + n * 8) * 2;
+        const bool valid = ok && (t0 + tt) < t_end;
+        r.k[i] = make_uint4(0, 0, 0, 0);
+        r.v[i] = make_uint4(0, 0, 0, 0);
+        if (valid) {
+          r.k[i] = load_nt_u4(p.k_cache + off);
+          r.v[i] = load_nt_u4(p.v_cache + off);
+        }
       }
     };
-    auto store_tile = [&](const TileRegs<KV8> &r) __attribute__((always_inline)) {
+    auto store_tile = [&](const TileRegs<KV8> &r) {
 #pragma unroll
       for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
-        // (a tile of an unmapped block is zeroed in LDS afterwards: a select on the loaded
-        // registers here would be hoisted to the top of the loop together with its wait)
-        const uint4 rk = r.k[i], rv = r.v[i];
         if (KV8) {
           const int tt = i * 8 + (lane >> 3);
           const int ch = (lane & 7) * 16;
           uint4 lo, hi;
-          fp8x16_to_bf16x16(rk, lo, hi);
+          fp8x16_to_bf16x16(r.k[i], lo, hi);
           *reinterpret_cast<uint4 *>(&Ks[tt][ch]) = lo;
           *reinterpret_cast<uint4 *>(&Ks[tt][ch + 8]) = hi;
-          fp8x16_to_bf16x16(rv, lo, hi);
+          fp8x16_to_bf16x16(r.v[i], lo, hi);
           *reinterpret_cast<uint4 *>(&Vs[tt][ch]) = lo;
           *reinterpret_cast<uint4 *>(&Vs[tt][ch + 8]) = hi;
         } else {
-          *reinterpret_cast<uint4 *>(&Ks[i * 4 + g][n * 8]) = rk;
-          *reinterpret_cast<uint4 *>(&Vs[i * 4 + g][n * 8]) = rv;
-        }
-      }
-      if (!r.ok) {  // wave-uniform, rare: what was read from block 0 must not reach the MFMAs
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          *reinterpret_cast<uint4 *>(&Ks[i * 4 + g][n * 8]) = make_uint4(0, 0, 0, 0);
-          *reinterpret_cast<uint4 *>(&Vs[i * 4 + g][n * 8]) = make_uint4(0, 0, 0, 0);
+          *reinterpret_cast<uint4 *>(&Ks[i * 4 + g][n * 8]) = r.k[i];
+          *reinterpret_cast<uint4 *>(&Vs[i * 4 + g][n * 8]) = r.v[i];
         }
       }
     };
@@ -272,33 +259,23 @@ void paged_decode_kernel(const DecodeParams p) {
 #pragma unroll
     for (int j = 0; j < PF; ++j) {
       const int tj = t_begin + j * kTile;
-      const bool real = tj < t_end;
-      const int blk0 = bt[(real ? tj : t_begin) / p.block_size];
+      if (tj < t_end) load_tile(tj, bt[tj / p.block_size], regs[j]);
       next_blk[j] = bt[min(tj + PF * kTile, t_end - 1) / p.block_size];
-      load_tile(tj, blk0, real, regs[j]);
-      // keep the tiles' loads in program order: the loop waits for the oldest tile by count
-      __builtin_amdgcn_sched_barrier(0);
     }
     for (int tg = t_begin; tg < t_end; tg += PF * kTile) {
 #pragma unroll
       for (int j = 0; j < PF; ++j) {
-        // no early exit for a tile past the end (t0 >= t_end, only in the last group of PF): every
-        // score of such a tile is masked, so it changes nothing, and the loop body stays free of
-        // branches around loads - with them the compiler waits for the whole load queue
         const int t0 = tg + j * kTile;
+        if (t0 >= t_end) break;  // uniform
         wave_lds_fence();  // previous tile's LDS reads are done
-        // e4m3: keep the conversion of this tile where it is; hoisted to the top of the loop it
-        // would take the wait for this tile's loads (the newest in the queue) with it
-        if constexpr (KV8) __builtin_amdgcn_sched_barrier(0);
         store_tile(regs[j]);
         wave_lds_fence();
         const bool tile_ok = regs[j].ok;
         const int tn = t0 + PF * kTile;
-        // the block-table fetch goes out before the tile's loads: it is waited for first, and a
-        // wait for the newest entry of the in-order queue would drain the tile loads behind it
-        const int blk_now = next_blk[j];
-        next_blk[j] = bt[min(tn + PF * kTile, t_end - 1) / p.block_size];
-        load_tile(tn, blk_now, tn < t_end, regs[j]);
+        if (tn < t_end) {
+          load_tile(tn, next_blk[j], regs[j]);
+          next_blk[j] = bt[min(tn + PF * kTile, t_end - 1) / p.block_size];
+        }
 
         // S^T = K . Q^T : lane (n, g) gets tokens g*4 + i of head n
         floatx4 s = floatx4{0.f, 0.f, 0.f, 0.f};
