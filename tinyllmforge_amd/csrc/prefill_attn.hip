@@ -118,28 +118,45 @@ void prefill_attn_kernel(const PrefillParams p) {
   constexpr int kChunks = KV8 ? 8 : 16;
   constexpr int kPasses = kBKV * kChunks / 256;
   uint4 kreg[kPasses], vreg[kPasses];
+  // Address arithmetic is kept off the vector ALU as far as possible (this kernel is VALU bound):
+  // everything that depends on the thread only is computed once, the tile's share is scalar.
+  constexpr int kRowsPerPass = 256 / kChunks;
+  const int trow = tid / kChunks, ch = tid % kChunks;
+  const int64_t k_thread = (static_cast<int64_t>(k_begin + trow) * p.k_stride + h * kPDh + ch * 8) * 2;
+  const int64_t v_thread = (static_cast<int64_t>(k_begin + trow) * p.v_stride + h * kPDh + ch * 8) * 2;
+  const int64_t cache_row_bytes = cache_row * (KV8 ? 1 : 2);
+  const int64_t paged_thread = static_cast<int64_t>(h) * kPDh * (KV8 ? 1 : 2) + ch * 16;
+  const int bs_shift = (p.block_size & (p.block_size - 1)) == 0 ? __builtin_ctz(p.block_size) : -1;
+  // Rows at or past kv_end are masked for every unit of this workgroup and get probability 0, so
+  // they only have to be finite: their loads re-read row kv_end-1 instead of being predicated.
   auto load_tile = [&](int kv0) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < kPasses; ++i) {
-      const int t = i * (256 / kChunks) + tid / kChunks;
-      const int ch = tid % kChunks;
-      const int tk = kv0 + t;
-      kreg[i] = make_uint4(0, 0, 0, 0);
-      vreg[i] = make_uint4(0, 0, 0, 0);
-      if (tk < kv_end) {
-        if (bt == nullptr) {
-          const int64_t ko = (static_cast<int64_t>(k_begin + tk) * p.k_stride + h * kPDh + ch * 8) * 2;
-          const int64_t vo = (static_cast<int64_t>(k_begin + tk) * p.v_stride + h * kPDh + ch * 8) * 2;
-          kreg[i] = *reinterpret_cast<const uint4 *>(p.k + ko);
-          vreg[i] = *reinterpret_cast<const uint4 *>(p.v + vo);
+      const int tk = kv0 + i * kRowsPerPass + trow;
+      if (bt == nullptr) {  // uniform
+        // scalar part of the row index, clamped per thread through a row delta
+        const int back = max(tk - (kv_end - 1), 0);  // rows to step back, 0 for a real row
+        const int64_t tile_k = static_cast<int64_t>(kv0 + i * kRowsPerPass) * p.k_stride * 2;
+        const int64_t tile_v = static_cast<int64_t>(kv0 + i * kRowsPerPass) * p.v_stride * 2;
+        kreg[i] = *reinterpret_cast<const uint4 *>(p.k + (k_thread + tile_k - back * (p.k_stride * 2)));
+        vreg[i] = *reinterpret_cast<const uint4 *>(p.v + (v_thread + tile_v - back * (p.v_stride * 2)));
+      } else {
+        const int tc = min(tk, kv_end - 1);
+        int bi, within;
+        if (bs_shift >= 0) {  // uniform: block sizes are powers of two in practice
+          bi = tc >> bs_shift;
+          within = tc & (p.block_size - 1);
         } else {
-          const int64_t blk = bt[tk / p.block_size];
-          if (blk >= 0 && blk < p.num_cache_blocks) {
-            const int64_t e = (blk * p.block_size + tk % p.block_size) * cache_row + h * kPDh;
-            const int64_t o = KV8 ? e + ch * 16 : (e + ch * 8) * 2;
-            kreg[i] = *reinterpret_cast<const uint4 *>(p.k + o);
-            vreg[i] = *reinterpret_cast<const uint4 *>(p.v + o);
-          }
+          bi = tc / p.block_size;
+          within = tc - bi * p.block_size;
+        }
+        const int64_t blk = bt[bi];
+        kreg[i] = make_uint4(0, 0, 0, 0);
+        vreg[i] = make_uint4(0, 0, 0, 0);
+        if (blk >= 0 && blk < p.num_cache_blocks) {  // an unmapped block reads as zeros
+          const int64_t o = (blk * p.block_size + within) * cache_row_bytes + paged_thread;
+          kreg[i] = *reinterpret_cast<const uint4 *>(p.k + o);
+          vreg[i] = *reinterpret_cast<const uint4 *>(p.v + o);
         }
       }
     }
@@ -147,8 +164,7 @@ void prefill_attn_kernel(const PrefillParams p) {
   auto store_tile = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < kPasses; ++i) {
-      const int t = i * (256 / kChunks) + tid / kChunks;
-      const int ch = tid % kChunks;
+      const int t = i * kRowsPerPass + trow;
       if (KV8) {
         uint4 lo, hi;
         fp8x16_to_bf16(kreg[i], lo, hi);
