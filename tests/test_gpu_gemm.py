@@ -45,6 +45,8 @@ SHAPES = [  # (M, N, K)
     # large-tile plans: ragged M and N with 5 K-tiles, an XCD patch of 4 columns with 3 K-tiles,
     # and the 128 x 64 tile with a split of K
     (2050, 8208, 320), (1100, 8192, 192), (512, 6144, 2048), (17, 1040, 64),
+    # one M-tile as tall as the batch against a wide N (130 -> 160 rows, 70 -> 96, 224 exactly)
+    (130, 16400, 256), (70, 16384, 192), (224, 16384, 128),
 ]
 
 
@@ -83,7 +85,7 @@ def test_w8a16_strided_activations_and_3d_input():
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 4096, 1024), (4, 151936, 1024), (512, 4096, 1024), (256, 6144, 4096), (2048, 3072, 1024), (77, 1024, 3072),
-                                   (2050, 8208, 320), (1100, 8192, 192), (512, 6144, 2048)])
+                                   (2050, 8208, 320), (1100, 8192, 192), (512, 6144, 2048), (130, 16400, 256), (200, 151936, 64)])
 def test_bf16_gemm(M, N, K):
     from tinyllmforge_amd import ops as P
     x = torch.randn(M, K, generator=g(M)).to(BF)
