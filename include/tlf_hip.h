@@ -192,6 +192,21 @@ int tlf_bf16_gemm(const void *x, int64_t x_stride, const void *w, void *y,
                   int32_t M, int32_t N, int32_t K,
                   void *workspace, size_t workspace_bytes, void *stream);
 
+/* gate_up projection fused with the activation: replaces MergedColumnParallelLinear.forward
+ * (layers/linear.py:82-83) followed by SiluAndMul.forward (layers/activation.py:11-14) in
+ * Qwen3MLP.forward (models/qwen3.py:123-130).
+ *
+ *   g = bf16(scale[..] * sum_k x[m,k] wq[.., k]),  u likewise
+ *   y[m, c] = bf16( bf16(silu(g[m, c])) * u[m, c] )          y: bf16 [M, N/2] contiguous
+ *
+ * wq / scale rows are INTERLEAVED: rows 16 j .. 16 j + 7 are gate channels 8 j .. 8 j + 7 and rows
+ * 16 j + 8 .. 16 j + 15 the matching up channels (N = 2 x intermediate size, N % 16 == 0), so that
+ * both halves of a product sit in one lane's accumulators.  Bit-identical to tlf_w8a16_gemm on
+ * the same interleaved weight followed by tlf_silu_and_mul on the de-interleaved result.
+ * Needs no workspace (K is never split across workgroups).  Other constraints as tlf_w8a16_gemm. */
+int tlf_w8a16_gemm_silu_mul(const void *x, int64_t x_stride, const void *wq, const float *scale,
+                            void *y, int32_t M, int32_t N, int32_t K, void *stream);
+
 /* Diagnostic, no counterpart in the reference, touches no GPU: the kernel plan the two GEMM entry
  * points would use for a shape.  plan8 = {tile channels, tile tokens, LDS stages, waves/SIMD budget,
  * K-groups per workgroup, split-K factor, K per split, N-tile columns per XCD patch}; tile 0 x 0

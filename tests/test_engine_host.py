@@ -234,3 +234,17 @@ def test_config_accepts_shape_names_and_dicts():
         Config("qwen3-8b", kvcache_block_size=100)
     with pytest.raises(AssertionError):
         Config("qwen3-8b", tensor_parallel_size=2)
+
+
+def test_gate_up_interleave_index_is_the_stated_permutation():
+    """Rows 16 j .. 16 j + 7 of the fused gate_up weight are gate channels 8 j .., rows 16 j + 8 .. 16 j + 15
+    the matching up channels (ops.gate_up_interleave_index)."""
+    import torch
+    from tinyllmforge_amd import ops as P
+    for n in (16, 32, 6144, 24576):
+        idx = P.gate_up_interleave_index(n)
+        assert sorted(idx.tolist()) == list(range(n))
+        half = n // 2
+        for j in range(0, n, 16):
+            assert idx[j:j + 8].tolist() == list(range(j // 2, j // 2 + 8))
+            assert idx[j + 8:j + 16].tolist() == list(range(half + j // 2, half + j // 2 + 8))

@@ -94,3 +94,23 @@ def test_bf16_gemm(M, N, K):
     absdot = (x.double().abs() @ w.double().abs().t()).float()
     got = P.bf16_linear(x.to(DEV), w.to(DEV))
     check(got, exact, exact.to(BF), absdot)
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 6144, 1024), (16, 2048, 4096), (130, 24576, 1024), (300, 6144, 2048),
+                                   (2048, 4096, 512), (70, 16384, 192), (33, 272, 64)])
+def test_w8a16_gemm_fused_silu_mul_equals_the_two_kernels(M, N, K):
+    """gate_up projection + SiLU-and-mul in one kernel (interleaved weight rows) is bit-identical to the
+    plain GEMM on the same weight followed by the activation kernel, and within tolerance of the oracle."""
+    from tinyllmforge_amd import ops as P
+    x = torch.randn(M, K, generator=g(M + 7)).to(BF)
+    wq, scale = make_w8(N, K, N)                       # natural order: [gate; up]
+    idx = P.gate_up_interleave_index(N)
+    wi, si = wq[idx].contiguous(), scale[idx].contiguous()
+    fused = P.w8a16_linear_silu_mul(x.to(DEV), wi.to(DEV), si.to(DEV))
+    assert fused.shape == (M, N // 2) and fused.dtype == BF
+    plain = P.w8a16_linear(x.to(DEV), wq.to(DEV), scale.to(DEV))          # natural layout
+    two = P.silu_and_mul(plain)
+    assert torch.equal(fused.view(torch.int16), two.view(torch.int16))
+    ref = O.silu_and_mul(O.w8a16_linear(x, wq, scale))
+    rel = ((fused.float().cpu() - ref.float()).norm() / ref.float().norm().clamp_min(1e-6)).item()
+    assert rel <= 2e-3, rel

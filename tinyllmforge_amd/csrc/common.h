@@ -35,6 +35,13 @@ __device__ __forceinline__ unsigned short float_to_bf16_bits(float f) {
   return __builtin_bit_cast(unsigned short, h);
 }
 
+// SiLU-and-mul with the eager rounding points of the reference (tinyvllm/layers/activation.py:11-14):
+// bf16(silu(g)) * u, the product rounded to bf16 by the caller's pack.  g and u are bf16 values.
+__device__ __forceinline__ float silu_mul_bf16(float g, float u) {
+  const float s = g / (1.0f + expf(-g));
+  return __fmul_rn(bf16_bits_to_float(float_to_bf16_bits(s)), u);
+}
+
 __device__ __forceinline__ unsigned int pack_bf16x2(float lo, float hi) {
   bf16x2 r;
   r[0] = static_cast<__bf16>(lo);

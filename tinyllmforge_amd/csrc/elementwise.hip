@@ -253,8 +253,7 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const unsigned short 
   unpack8(*reinterpret_cast<const uint4 *>(xr + inter + c * 8), u);
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    const float s = g[i] / (1.0f + expf(-g[i]));
-    o[i] = __fmul_rn(bf16_bits_to_float(float_to_bf16_bits(s)), u[i]);
+    o[i] = silu_mul_bf16(g[i], u[i]);
   }
   *reinterpret_cast<uint4 *>(y + r * inter + c * 8) = pack8(o);
 }

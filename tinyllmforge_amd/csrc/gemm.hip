@@ -48,6 +48,7 @@ struct GemmParams {
   int32_t splits;
   int32_t m_tiles, n_tiles;
   int32_t group_n;  // N-tile columns walked together by one XCD (direct-to-LDS kernel)
+  int32_t act;      // 1: SiLU-and-mul epilogue over interleaved gate/up channels, y is [M, N/2]
 };
 
 // BN x BM output tile per workgroup (BN output channels, BM tokens), 4 waves as WAVES_N x WAVES_M.
@@ -64,6 +65,38 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
     if (m >= p.M) continue;
 #pragma unroll
     for (int i = 0; i < TN; ++i) {
+      if (p.act) {
+        // channels come in groups of 16 = 8 gate rows then the 8 matching up rows, so this lane's
+        // registers q = 0, 2 hold gate values and q = 1, 3 the up values of the same 4 channels
+#pragma unroll
+        for (int q = 0; q < 4; q += 2) {
+          const int n = n0 + wn * WN + i * 32 + q * 8 + kg * 4;  // first gate row of the four
+          if (n >= p.N) continue;
+          float gt[4], up[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            gt[e] = acc[i][j][q * 4 + e];
+            up[e] = acc[i][j][(q + 1) * 4 + e];
+          }
+          if (W8) {
+            const float4 sg = *reinterpret_cast<const float4 *>(p.scale + n);
+            const float4 su = *reinterpret_cast<const float4 *>(p.scale + n + 8);
+            gt[0] *= sg.x; gt[1] *= sg.y; gt[2] *= sg.z; gt[3] *= sg.w;
+            up[0] *= su.x; up[1] *= su.y; up[2] *= su.z; up[3] *= su.w;
+          }
+          float o[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e)  // both factors rounded to bf16 first, as the unfused sequence does
+            o[e] = silu_mul_bf16(bf16_bits_to_float(float_to_bf16_bits(gt[e])),
+                                 bf16_bits_to_float(float_to_bf16_bits(up[e])));
+          uint2 st;
+          st.x = pack_bf16x2(o[0], o[1]);
+          st.y = pack_bf16x2(o[2], o[3]);
+          const int c = (n0 + wn * WN + i * 32) / 2 + (q / 2) * 8 + kg * 4;  // output channel
+          *reinterpret_cast<uint2 *>(p.y + static_cast<int64_t>(m) * (p.N / 2) + c) = st;
+        }
+        continue;
+      }
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int n = n0 + wn * WN + i * 32 + q * 8 + kg * 4;
@@ -89,7 +122,6 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
   }
 }
 
-// ---------------------------------------------------------------------------
 // Tiled kernel: global_load_lds_dwordx4 copies each lane's 16 bytes from global memory
 // straight into LDS (the wave's 64 pieces land contiguously at a wave-uniform LDS base), so a K-tile
 // costs no staging registers, no ds_write and - for int8 weights - half the LDS bytes: W stays
@@ -571,6 +603,28 @@ __global__ __launch_bounds__(512) void skinny_gemm_kernel(const GemmParams p) {
       const float4 sc = *reinterpret_cast<const float4 *>(p.scale + n);
       s.x *= sc.x; s.y *= sc.y; s.z *= sc.z; s.w *= sc.w;
     }
+    if (p.act) {
+      // a 16-channel tile is 8 gate rows then the 8 matching up rows: lanes 0..31 hold gate values,
+      // lane l + 32 the up values of the same 4 channels; the gate lanes finish the pair
+      if (l >= 32) continue;
+      float4 u = *reinterpret_cast<const float4 *>(&red[0][tile][l + 32][0]);
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) {
+        const float4 v = *reinterpret_cast<const float4 *>(&red[w][tile][l + 32][0]);
+        u.x += v.x; u.y += v.y; u.z += v.z; u.w += v.w;
+      }
+      if (W8) {
+        const float4 sc = *reinterpret_cast<const float4 *>(p.scale + n + 8);
+        u.x *= sc.x; u.y *= sc.y; u.z *= sc.z; u.w *= sc.w;
+      }
+      auto rb = [](float v) { return bf16_bits_to_float(float_to_bf16_bits(v)); };
+      uint2 st;
+      st.x = pack_bf16x2(silu_mul_bf16(rb(s.x), rb(u.x)), silu_mul_bf16(rb(s.y), rb(u.y)));
+      st.y = pack_bf16x2(silu_mul_bf16(rb(s.z), rb(u.z)), silu_mul_bf16(rb(s.w), rb(u.w)));
+      const int c = (n0 + t * 16) / 2 + (l >> 4) * 4;
+      *reinterpret_cast<uint2 *>(p.y + static_cast<int64_t>(token) * (p.N / 2) + c) = st;
+      continue;
+    }
     uint2 st;
     st.x = pack_bf16x2(s.x, s.y);
     st.y = pack_bf16x2(s.z, s.w);
@@ -710,7 +764,7 @@ inline int skinny_max_m() {
 template <bool W8>
 int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *scale, void *y,
                 int32_t M, int32_t N, int32_t K, void *workspace, size_t workspace_bytes,
-                hipStream_t stream, int32_t *plan_out = nullptr) {
+                hipStream_t stream, int32_t *plan_out = nullptr, int32_t act = 0) {
   const bool dry = plan_out != nullptr;
   GemmParams p;
   p.x = static_cast<const unsigned char *>(x);
@@ -720,6 +774,7 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   p.y = static_cast<unsigned short *>(y);
   p.partial = nullptr;
   p.M = M; p.N = N; p.K = K;
+  p.act = act;
   if (M <= skinny_max_m()) {
     p.k_per_split = K; p.splits = 1; p.m_tiles = 1; p.n_tiles = 1; p.group_n = 1;
     if (dry) {
@@ -731,6 +786,10 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   }
   GemmPlan g = plan_gemm(M, N, K, W8);
   plan_override(g, K);
+  if (act) {  // the activation needs whole sums: no split of K across workgroups
+    g.splits = 1;
+    g.k_per_split = K;
+  }
   if (g.kgroups > 1) {
     // every split must hand each wave set the same whole number of K-tiles
     const int ktiles = K / kBK;
@@ -857,4 +916,16 @@ extern "C" int tlf_gemm_plan(int32_t M, int32_t N, int32_t K, int32_t w8, int32_
   if (M <= 0 || N <= 0 || K <= 0 || K % kBK || N % 16) return TLF_E_SHAPE;
   return w8 ? launch_gemm<true>(nullptr, K, nullptr, nullptr, nullptr, M, N, K, nullptr, 0, nullptr, plan8)
             : launch_gemm<false>(nullptr, K, nullptr, nullptr, nullptr, M, N, K, nullptr, 0, nullptr, plan8);
+}
+
+extern "C" int tlf_w8a16_gemm_silu_mul(const void *x, int64_t x_stride, const void *wq,
+                                       const float *scale, void *y, int32_t M, int32_t N, int32_t K,
+                                       void *stream) {
+  if (M == 0) return TLF_OK;
+  const int rc = check_gemm_args(x, x_stride, wq, y, M, N, K);
+  if (rc != TLF_OK) return rc;
+  if (!scale) return TLF_E_NULL;
+  if (reinterpret_cast<uintptr_t>(scale) & 15u) return TLF_E_ALIGN;
+  return launch_gemm<true>(x, x_stride, wq, scale, y, M, N, K, nullptr, 0,
+                           static_cast<hipStream_t>(stream), nullptr, 1);
 }

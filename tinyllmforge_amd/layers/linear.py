@@ -88,6 +88,29 @@ class MergedColumnParallelLinear(ColumnParallelLinear):
         self.output_sizes = output_sizes
         super().__init__(input_size, sum(output_sizes), bias=bias)
 
+    def quantize_(self):
+        """int8 + scale; a gate/up pair is also re-ordered for the fused projection + SiLU-and-mul
+        kernel (``ops.gate_up_interleave_index``), which ``forward_silu_mul`` then uses."""
+        super().quantize_()
+        if len(self.output_sizes) == 2 and self.output_sizes[0] == self.output_sizes[1] \
+                and sum(self.output_sizes) % 16 == 0 and self.bias is None:
+            idx = ops.gate_up_interleave_index(sum(self.output_sizes), self.qweight.device)
+            self.qweight = self.qweight[idx].contiguous()
+            self.qscale = self.qscale[idx].contiguous()
+            self.interleaved = True
+        return self
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if getattr(self, "interleaved", False):
+            raise RuntimeError("this gate_up weight is interleaved for the fused kernel: call forward_silu_mul")
+        return super().forward(x)
+
+    def forward_silu_mul(self, x: torch.Tensor) -> torch.Tensor:
+        """``SiluAndMul()(self(x))`` (activation.py:11-14 after linear.py:82-83), fused when quantised."""
+        if getattr(self, "interleaved", False):
+            return ops.w8a16_linear_silu_mul(x, self.qweight, self.qscale)
+        return ops.silu_and_mul(super().forward(x))
+
     def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor, loaded_shard_id: int):
         offset = sum(self.output_sizes[:loaded_shard_id]) // self.tp_size
         size = self.output_sizes[loaded_shard_id] // self.tp_size

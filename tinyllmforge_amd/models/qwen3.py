@@ -69,7 +69,8 @@ class Qwen3MLP(nn.Module):
         self.act_fn = SiluAndMul()
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return self.down_proj(self.act_fn(self.gate_up_proj(x)))
+        # gate_up projection and activation in one kernel when the weights are int8 (qwen3.py:123-130)
+        return self.down_proj(self.gate_up_proj.forward_silu_mul(x))
 
 
 class Qwen3DecoderLayer(nn.Module):

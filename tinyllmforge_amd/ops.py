@@ -207,6 +207,33 @@ def w8a16_linear(x, wq, scale):
     return y.view(*x.shape[:-1], N)
 
 
+def gate_up_interleave_index(n: int, device=None):
+    """Row order of the fused gate_up weight: rows ``16 j .. 16 j + 7`` = gate channels ``8 j ..``, rows
+    ``16 j + 8 .. 16 j + 15`` = the matching up channels; ``n`` = 2 x intermediate size.  ``w[idx]``
+    interleaves a ``[gate; up]`` stacked weight (or scale)."""
+    assert n % 16 == 0
+    half = n // 2
+    j = torch.arange(n, device=device)
+    group, r = j // 16, j % 16
+    return torch.where(r < 8, group * 8 + r, half + group * 8 + (r - 8))
+
+
+def w8a16_linear_silu_mul(x, wq_interleaved, scale_interleaved):
+    """``silu(gate) * up`` of the int8 gate_up projection in one kernel; weight rows interleaved as
+    ``gate_up_interleave_index`` says.  Returns ``[..., N / 2]``."""
+    lib = _lib.load()
+    _need(x, BF16, "x"); _need(wq_interleaved, torch.int8, "wq"); _need(scale_interleaved, torch.float32, "scale")
+    assert x.stride(-1) == 1 and wq_interleaved.is_contiguous()
+    x2 = x.reshape(-1, x.shape[-1])
+    M, K = x2.shape
+    N = wq_interleaved.shape[0]
+    y = torch.empty(M, N // 2, dtype=BF16, device=x.device)
+    check(lib.tlf_w8a16_gemm_silu_mul(x2.data_ptr(), x2.stride(0), wq_interleaved.data_ptr(),
+                                      scale_interleaved.data_ptr(), y.data_ptr(), M, N, K, _stream()),
+          "tlf_w8a16_gemm_silu_mul")
+    return y.view(*x.shape[:-1], N // 2)
+
+
 def bf16_linear(x, w):
     lib = _lib.load()
     _need(x, BF16, "x"); _need(w, BF16, "w")
