@@ -715,6 +715,10 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
     g.bn = 128; g.bm = 64; g.stages = 2; g.occ = 3;
   } else if (tiles(128, 128) < 1024) {
     g.bn = 128; g.bm = 128; g.stages = 3; g.occ = 2;
+  } else if (w8 && K >= 8192) {
+    // long K (down projections): the square tile moves the fewest bytes per flop (measured 5-6 %
+    // faster than 256 x 128 on 4096 x 12288 and 5120 x 25600)
+    g.bn = 256; g.bm = 256; g.stages = 3; g.occ = 1;
   } else if (w8) {
     g.bn = 256; g.bm = 128; g.stages = 2; g.occ = 2;  // 64 KB of LDS: two workgroups per CU
   } else {
