@@ -125,9 +125,10 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
 // Tiled kernel: global_load_lds_dwordx4 copies each lane's 16 bytes from global memory
 // straight into LDS (the wave's 64 pieces land contiguously at a wave-uniform LDS base), so a K-tile
 // costs no staging registers, no ds_write and - for int8 weights - half the LDS bytes: W stays
-// int8 in LDS and is converted to bf16 after the fragment read.  Three LDS stages, each its own
-// __shared__ object (the compiler then tracks which outstanding copies a ds_read has to wait
-// for per object): while tile t is computed, the copies of tiles t+1 and t+2 are in flight.
+// int8 in LDS and is converted to bf16 after the fragment read.  NS LDS stages carved out of
+// one pool: with three, the copies of tiles t+1 and t+2 are in flight while tile t is computed;
+// two suffice where the copies are L2 hits, four and more help where few workgroups stream
+// weights from HBM.
 //
 // LDS rows are unpadded (a wave's copy is contiguous), conflicts are avoided by an XOR swizzle of
 // the 16-byte pieces instead: piece c of a 128-byte bf16 row R sits at position c ^ ((R>>1)&7),
@@ -137,7 +138,6 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
 // int8 weights: lane (r, kg) reads 16 consecutive K values of channel r with one ds_read_b128 and
 // feeds them to two MFMAs; the K index inside an MFMA is only a summation label, so the x operand
 // of those two MFMAs is read with the same labelling (pieces 2c and 2c+1 of the x row).
-#define TLF_GPTR(p) ((const __attribute__((address_space(1))) void *)(p))
 #define TLF_LPTR(p) ((__attribute__((address_space(3))) void *)(p))
 // Workgroup barrier for the copy pipeline: wait until at most N of this wave's copies are still
 // in flight and its LDS reads have returned, then s_barrier.  Written as one asm block: a
@@ -446,6 +446,9 @@ void gemm_dlds_kernel(const GemmParams p) {
 #undef TLF_DL_AFTER_GROUP
 #undef TLF_DL_ISSUE_SETUP
 #undef TLF_DL_COPY
+#undef TLF_DL_LDSADDR
+#undef TLF_DL_BARRIER
+#undef TLF_LPTR
 
 // Sum the split-K partials, apply the channel scale, round once to bf16.
 template <bool W8>
