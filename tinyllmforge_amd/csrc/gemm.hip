@@ -47,13 +47,13 @@ struct GemmParams {
   int32_t k_per_split;
   int32_t splits;
   int32_t m_tiles, n_tiles;
-  int32_t group_n;  // N-tile columns walked together by one XCD (direct-to-LDS kernel)
+  int32_t group_n;  // N-tile columns walked together by one XCD
   int32_t act;      // 1: SiLU-and-mul epilogue over interleaved gate/up channels, y is [M, N/2]
 };
 
-// BN x BM output tile per workgroup (BN output channels, BM tokens), 4 waves as WAVES_N x WAVES_M.
-// Epilogue shared by the tiled kernels: scale (W8), round once to bf16, 8-byte stores;
-// or fp32 partials when K is split.
+// Epilogue of the tiled kernel (BN output channels x BM tokens per workgroup, waves laid out as
+// WAVES_N x WAVES_M): scale (W8), round once to bf16, 8-byte stores; or fp32 partials when K is
+// split across workgroups; or the fused SiLU-and-mul over interleaved gate/up channels.
 template <int TN, int TM, int WN, int WM, bool W8>
 __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&acc)[TN][TM], int m0,
                                               int n0, int wn, int wm, int r, int kg, int split) {
@@ -265,7 +265,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
     TLF_DL_COMPUTE(XS, WS)                        \
   }
 
-// NS = LDS stages (2 or 3), OCC = waves per SIMD the register budget is cut for.
+// NS = LDS stages (2 ... 8), OCC = waves per SIMD the register budget is cut for.
 // KG = K-groups: the workgroup holds KG independent sets of WAVES_N x WAVES_M waves; set g runs the
 // pipeline over its own 1/KG of the K range in its own LDS stages and the sets' accumulators are
 // summed through LDS at the end.  A latency-bound problem (few tiles, long K) then takes 1/KG of
