@@ -47,6 +47,8 @@ SHAPES = [  # (M, N, K)
     (2050, 8208, 320), (1100, 8192, 192), (512, 6144, 2048), (17, 1040, 64),
     # one M-tile as tall as the batch against a wide N (130 -> 160 rows, 70 -> 96, 224 exactly)
     (130, 16400, 256), (70, 16384, 192), (224, 16384, 128),
+    # one M-tile, 64 channels, two wave sets splitting K (decode-size batch, moderate N)
+    (150, 1024, 12288), (140, 6144, 4096), (90, 1040, 8320),
 ]
 
 

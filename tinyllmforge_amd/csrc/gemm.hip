@@ -275,7 +275,7 @@ __global__ __launch_bounds__(WAVES_N * WAVES_M * KG * 64) __attribute__((amdgpu_
 void gemm_dlds_kernel(const GemmParams p) {
   static_assert(NS >= 2 && NS <= 8, "2 to 8 stages");
   constexpr int NW = WAVES_N * WAVES_M;       // waves of one set
-  static_assert(NW == 4 || NW == 8, "4 or 8 waves");  // 8: two waves share each SIMD (not faster in the sweeps)
+  static_assert(NW == 2 || NW == 4 || NW == 8, "2, 4 or 8 waves");  // 8: two waves share each SIMD (not faster in the sweeps)
   static_assert(NW * KG <= 16, "at most 1024 threads");
   constexpr int WN = BN / WAVES_N, WM = BM / WAVES_M;
   constexpr int TN = WN / 32, TM = WM / 32;
@@ -693,6 +693,14 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
     // each CU once; four waves side by side along N.  Measured on 24576 x 4096 at M = 130:
     // 62 -> 49 us (int8), 56 -> 40 us (bf16); LM head 342 -> 300 us.
     g.bn = 128; g.bm = (M + 31) / 32 * 32; g.stages = 3; g.occ = 2; g.wn = 4;
+  } else if (w8 && M > 64 && M <= 160 && (N + 63) / 64 <= 128 && ktiles % 2 == 0 &&
+             (ktiles > 64 || (M > 128 && tiles(64, 64) > 256))) {
+    // decode-size batch, moderate N: again one M-tile as tall as the batch, here 64 channels wide
+    // with two waves per set and two sets splitting K inside the workgroup, three stages, plus a
+    // split of K across workgroups.  Measured at M = 130 (M = 96): 6144 x 4096 25 -> 20 us,
+    // 4096 x 12288 40 -> 30 us (29 -> 24 us); 4096 x 4096 is better off below.
+    g.bn = 64; g.bm = (M + 31) / 32 * 32; g.stages = 3; g.occ = 2; g.wn = 2; g.kgroups = 2;
+    splits = ktiles >= 128 ? 4 : 2;
   } else if (tiles(64, 64) <= 512) {
     g.bn = 64; g.bm = 64; g.stages = 2; g.occ = 4;
     splits = pow2_floor(1024 / tiles(64, 64));
@@ -851,6 +859,9 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   TLF_TILE(128, 192, 4, 1, 3, 2)
   TLF_TILE(128, 224, 4, 1, 3, 2)
   if constexpr (W8) {  // these fit LDS with int8 weights only
+    TLF_TILE_KG(64, 96, 2, 1, 3, 2, 2)   // one M-tile, 64 channels, two sets of two waves
+    TLF_TILE_KG(64, 128, 2, 1, 3, 2, 2)
+    TLF_TILE_KG(64, 160, 2, 1, 3, 2, 2)
     TLF_TILE_KG(64, 64, 2, 2, 3, 4, 4)
     TLF_TILE(256, 256, 2, 2, 3, 1)
   }
