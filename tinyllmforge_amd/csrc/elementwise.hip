@@ -27,11 +27,14 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(
   const int64_t out_off = safe_row * cols;
 
   float v[MAXC][8];
+  uint4 pw[MAXC];  // the weights do not depend on the row: fetched together with it, not after the reduction
   float ss = 0.f;
 #pragma unroll
   for (int c = 0; c < MAXC; ++c) {
     const int chunk = sub + c * TPR;
+    pw[c] = make_uint4(0, 0, 0, 0);
     if (active && chunk < nchunks) {
+      pw[c] = *reinterpret_cast<const uint4 *>(weight + chunk * 8);
       uint4 p = *reinterpret_cast<const uint4 *>(xr + chunk * 8);
       unpack8(p, v[c]);
       if (ADD) {
@@ -66,8 +69,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(
     const int chunk = sub + c * TPR;
     if (active && chunk < nchunks) {
       float w[8];
-      uint4 pw = *reinterpret_cast<const uint4 *>(weight + chunk * 8);
-      unpack8(pw, w);
+      unpack8(pw[c], w);
       float o[8];
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
