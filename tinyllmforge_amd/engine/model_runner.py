@@ -149,6 +149,8 @@ class ModelRunner:
     def prepare_sample(self, seqs):
         t = np.asarray([s.temperature for s in seqs], dtype=np.float32)
         self._all_greedy = bool((t == 0).all())
+        if self._all_greedy:
+            return None                      # the greedy kernel does not read temperatures
         return torch.from_numpy(t).to(self.device, non_blocking=True)
 
     # ------------------------------------------------------------------ forward
@@ -174,7 +176,41 @@ class ModelRunner:
         self.graphs[gbs].replay()
         return self.model.compute_logits(gv["outputs"][:bs])
 
+    @torch.inference_mode()
+    def run_decode_graph(self, seqs):
+        """Decode step through a captured graph: the integer inputs (I.decode_inputs, the same function the
+        eager path uploads) are written straight into the pinned mirror of the graph's static buffers,
+        padding rows get slot -1 (no cache write) and length 0 (no cache read), one H2D copy, replay."""
+        bs = len(seqs)
+        gbs = next(x for x in self.graph_bs if x >= bs)
+        d = I.decode_inputs(seqs, self.block_size, self.config.decode_position_quirk)
+        h = self.graph_host
+        h["input_ids"][:bs] = d["input_ids"]
+        h["positions"][:bs] = d["positions"]
+        h["slot_mapping"][:bs] = d["slot_mapping"]
+        h["context_lens"][:bs] = d["context_lens"]
+        w = d["block_tables"].shape[1]
+        h["block_tables"][:bs, :w] = d["block_tables"]
+        if gbs != bs:
+            h["input_ids"][bs:gbs] = 0
+            h["positions"][bs:gbs] = 0
+            h["slot_mapping"][bs:gbs] = -1
+            h["context_lens"][bs:gbs] = 0
+        self.graph_pack_dev.copy_(self.graph_pack_host, non_blocking=True)
+        set_context(False)
+        self.graphs[gbs].replay()
+        return self.model.compute_logits(self.graph_vars["outputs"][:bs])
+
     def run(self, seqs, is_prefill):
+        use_graph = (not is_prefill and not self.enforce_eager and self.graph_bs
+                     and len(seqs) <= self.graph_bs[-1]
+                     and max(len(s.block_table) for s in seqs) <= self.graph_max_blocks)
+        if use_graph:
+            temperatures = self.prepare_sample(seqs)
+            logits = self.run_decode_graph(seqs)
+            token_ids = self.sampler(logits, temperatures, self._all_greedy).tolist()
+            reset_context()
+            return token_ids
         input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
         temperatures = self.prepare_sample(seqs)
         logits = self.run_model(input_ids, positions, is_prefill)
@@ -192,14 +228,29 @@ class ModelRunner:
         max_bs = min(cfg.max_num_seqs, 512)
         max_blocks = (cfg.max_model_len + self.block_size - 1) // self.block_size
         dev = self.device
-        gv = dict(
-            input_ids=torch.zeros(max_bs, dtype=torch.int64, device=dev),
-            positions=torch.zeros(max_bs, dtype=torch.int64, device=dev),
-            slot_mapping=torch.full((max_bs,), -1, dtype=torch.int32, device=dev),
-            context_lens=torch.zeros(max_bs, dtype=torch.int32, device=dev),
-            block_tables=torch.zeros(max_bs, max_blocks, dtype=torch.int32, device=dev),
-            outputs=torch.zeros(max_bs, hf.hidden_size, dtype=hf.torch_dtype, device=dev),
-        )
+        # The static integer inputs of the graphs live in ONE device allocation mirrored by ONE pinned
+        # host buffer of the same layout: a decode step writes the host mirror in place (padding
+        # rows included) and issues a single H2D copy - no per-step staging allocation, no
+        # device-side copies or fills between the replays.
+        layout, off = {}, 0
+        for name, dt, shape in (("input_ids", torch.int64, (max_bs,)), ("positions", torch.int64, (max_bs,)),
+                                ("slot_mapping", torch.int32, (max_bs,)), ("context_lens", torch.int32, (max_bs,)),
+                                ("block_tables", torch.int32, (max_bs, max_blocks))):
+            nbytes = int(np.prod(shape)) * torch.empty(0, dtype=dt).element_size()
+            layout[name] = (off, nbytes, dt, shape)
+            off += (nbytes + 15) // 16 * 16
+        self.graph_pack_dev = torch.zeros(off, dtype=torch.uint8, device=dev)
+        self.graph_pack_host = torch.zeros(off, dtype=torch.uint8, pin_memory=True)
+        host_np = self.graph_pack_host.numpy()
+        np_dt = {torch.int64: np.int64, torch.int32: np.int32}
+        gv, self.graph_host = {}, {}
+        for name, (o, nbytes, dt, shape) in layout.items():
+            gv[name] = self.graph_pack_dev[o:o + nbytes].view(dt).view(*shape)
+            self.graph_host[name] = host_np[o:o + nbytes].view(np_dt[dt]).reshape(shape)
+        self.graph_host["slot_mapping"][:] = -1
+        self.graph_pack_dev.copy_(self.graph_pack_host)
+        gv["outputs"] = torch.zeros(max_bs, hf.hidden_size, dtype=hf.torch_dtype, device=dev)
+        self.graph_max_blocks = max_blocks
         self.graph_bs = [b for b in (1, 2, 4, 8) if b <= max_bs] + list(range(16, max_bs + 1, 16))
         pool = None
         for bs in reversed(self.graph_bs):
