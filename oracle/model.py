@@ -18,13 +18,21 @@ from . import ops as O
 
 
 class OracleQwen3:
-    def __init__(self, cfg: dict, params: dict, exact: bool = True):
+    def __init__(self, cfg: dict, params: dict, exact: bool = True, w8a16: bool = False):
         """``params``: ``{name: tensor}`` with the reference's packed parameter names
         (``model.layers.N.self_attn.qkv_proj.weight`` ...).  ``exact=False`` runs the linears as the
-        reference does on a CPU (``F.linear`` in bf16, no fp64 copies): used for timing only."""
+        reference does on a CPU (``F.linear`` in bf16, no fp64 copies): used for timing only.
+        ``w8a16=True`` (build-defined, not in the reference): the four projections of every layer are
+        quantised with ``ops.quantize_w8`` and run through ``ops.w8a16_linear``; embedding and LM head
+        stay bf16."""
         self.cfg = dict(cfg)
         self.exact = exact
         self.p = {k: v.detach().cpu() for k, v in params.items()}
+        self.q8 = {}
+        if w8a16:
+            for k in list(self.p):
+                if k.endswith("proj.weight"):
+                    self.q8[k] = O.quantize_w8(self.p[k])
         self.p64 = {}
         if exact:
             self.p64 = {k: v.double() for k, v in self.p.items() if k.endswith("proj.weight") or "embed_tokens" in k
@@ -40,6 +48,8 @@ class OracleQwen3:
             self.p64["lm_head.weight"] = self.p64["model.embed_tokens.weight"]
 
     def lin(self, x, name):
+        if name in self.q8:
+            return O.w8a16_linear(x, *self.q8[name])
         if not self.exact:
             return O.linear(x, self.p[name])
         return (x.double() @ self.p64[name].t()).to(x.dtype)

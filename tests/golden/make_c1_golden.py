@@ -1,6 +1,7 @@
 """Writes tests/golden/c1_greedy.json: greedy token ids of the CPU oracle on BASELINE config 1.
 
-    python tests/golden/make_c1_golden.py
+    python tests/golden/make_c1_golden.py            # bf16 linears, 32 tokens -> c1_greedy.json
+    python tests/golden/make_c1_golden.py --w8a16    # int8 projections, 8 tokens -> c1_w8a16_greedy.json
 
 Config 1: Qwen3-0.6B-shaped decoder (28 layers, hidden 1024, 16 query / 8 KV heads, head_dim 128,
 intermediate 3072, vocab 151936, RMSNorm eps 1e-6 + q/k-norm, RoPE theta 1e6, tied embeddings),
@@ -48,17 +49,19 @@ def c1_prompts():
 
 
 def main():
+    w8 = "--w8a16" in sys.argv
     cfg = c1_config()
     t0 = time.time()
     params = c1_params(cfg)
-    oracle = OracleQwen3(vars(cfg), params)
+    oracle = OracleQwen3(vars(cfg), params, w8a16=w8)
     prompts = c1_prompts()
-    ids, margins, topk = greedy_generate(oracle, prompts, max_tokens=32, block_size=256)
-    out = dict(config="BASELINE.json configs[0]", seed=0, prompt_first_tokens=[p[:4] for p in prompts],
+    ids, margins, topk = greedy_generate(oracle, prompts, max_tokens=8 if w8 else 32, block_size=256)
+    out = dict(config="BASELINE.json configs[0]" + (" with int8 per-channel projection weights" if w8 else ""),
+               seed=0, prompt_first_tokens=[p[:4] for p in prompts],
                token_ids=ids, top2_margin=[[round(m, 6) for m in row] for row in margins],
                top4_ids=[t[0] for t in topk], top4_logits=[t[1] for t in topk],
                bf16_ulp_note="margins are differences of bf16 logits; 0.0 is an exact tie (first index wins)")
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "c1_greedy.json")
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "c1_w8a16_greedy.json" if w8 else "c1_greedy.json")
     with open(path, "w") as f:
         json.dump(out, f)
     print("wrote", path, "in %.1f s" % (time.time() - t0))

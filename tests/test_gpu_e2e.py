@@ -66,27 +66,23 @@ def test_c1_greedy_token_ids_free_running(llm_c1, golden):
     assert st["prefill_steps"] == 1 and st["prefill_tokens"] == 516 and st["decode_steps"] == 31
 
 
-def test_c1_teacher_forced_every_step(llm_c1, golden):
-    """Feed the oracle's tokens and check all 4 x 32 decisions and logits of the HIP path.
-
-    After 28 bf16 layers the logits of the two pipelines agree to within 3 bf16 ulp (measured: 2);
-    a decision is therefore required to be identical whenever the oracle's margin exceeds 2 ulp, and
-    must otherwise fall on one of the oracle's candidates inside that band.
-    """
+def teacher_forced(llm, golden, steps):
+    """Feed the oracle's tokens through the engine's runner and check every decision and the logits of
+    the oracle's best candidates.  Returns (identical decisions, near-tie steps, worst |logit diff|)."""
     from tinyllmforge_amd.engine.sequence import Sequence
     from tinyllmforge_amd.sampling_params import SamplingParams
-    runner, sch = llm_c1.model_runner, llm_c1.scheduler
-    sp = SamplingParams(temperature=0.0, max_tokens=32, ignore_eos=True)
+    from tinyllmforge_amd.utils.context import reset_context
+    runner, sch = llm.model_runner, llm.scheduler
+    sp = SamplingParams(temperature=0.0, max_tokens=steps, ignore_eos=True)
     seqs0 = [Sequence(p, sp) for p in c1_prompts()]
     for s in seqs0:
         sch.add(s)
     same, tied, worst = 0, 0, 0.0
-    for step in range(32):
+    for step in range(steps):
         seqs, is_prefill = sch.schedule()
         assert [q.seq_id for q in seqs] == [q.seq_id for q in seqs0] and is_prefill == (step == 0)
         ids, pos = runner.prepare_prefill(seqs) if is_prefill else runner.prepare_decode(seqs)
         logits = runner.run_model(ids, pos, is_prefill).float().cpu()
-        from tinyllmforge_amd.utils.context import reset_context
         reset_context()
         choice = logits.argmax(-1).tolist()
         for s in range(4):
@@ -104,8 +100,36 @@ def test_c1_teacher_forced_every_step(llm_c1, golden):
             same += choice[s] == want
         sch.postprocess(seqs, [golden["token_ids"][s][step] for s in range(4)])
     assert sch.is_finished()
+    return same, tied, worst
+
+
+def test_c1_teacher_forced_every_step(llm_c1, golden):
+    """Feed the oracle's tokens and check all 4 x 32 decisions and logits of the HIP path.
+
+    After 28 bf16 layers the logits of the two pipelines agree to within 3 bf16 ulp (measured: 2);
+    a decision is therefore required to be identical whenever the oracle's margin exceeds 2 ulp, and
+    must otherwise fall on one of the oracle's candidates inside that band.
+    """
+    same, tied, worst = teacher_forced(llm_c1, golden, 32)
     print(f"teacher-forced: {same}/128 decisions identical, {tied} near-tie steps, max |logit diff| {worst:.4f}")
     assert same >= 128 - tied
+
+
+def test_c1_w8a16_teacher_forced_against_the_quantised_oracle():
+    """The same check for the weight-only int8 model (int8 GEMMs, fused gate_up + SiLU-and-mul): 4 x 8
+    decisions against tests/golden/c1_w8a16_greedy.json, written by the oracle with quantised projections."""
+    from tinyllmforge_amd import LLM
+    with open(os.path.join(os.path.dirname(GOLDEN), "c1_w8a16_greedy.json")) as f:
+        gold8 = json.load(f)
+    llm = LLM("qwen3-0.6b", max_model_len=1024, max_num_batched_tokens=4096, max_num_seqs=8,
+              num_kvcache_blocks=48, enforce_eager=False, seed=0, quantization="w8a16")
+    try:
+        assert getattr(llm.model_runner.model.model.layers[0].mlp.gate_up_proj, "interleaved", False)
+        same, tied, worst = teacher_forced(llm, gold8, 8)
+        print(f"w8a16 teacher-forced: {same}/32 decisions identical, {tied} near-tie steps, max |logit diff| {worst:.4f}")
+        assert same >= 32 - tied
+    finally:
+        llm.exit()
 
 
 def test_c1_eager_equals_graph_and_rerun_hits_prefix_cache(llm_c1, golden):

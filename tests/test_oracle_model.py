@@ -72,18 +72,39 @@ def test_decode_position_quirk_changes_the_rotation():
     assert not torch.equal(outs[0], outs[1])
 
 
-@pytest.mark.skipif(not os.path.exists(os.path.join(os.path.dirname(__file__), "golden", "c1_greedy.json")), reason="no fixture")
-def test_c1_fixture_first_steps_reproduce():
-    """Recompute prefill + 2 decode steps of config 1 with the oracle (about 20 s) and compare with the fixture."""
+@pytest.mark.parametrize("fixture,w8a16,steps", [("c1_greedy.json", False, 3), ("c1_w8a16_greedy.json", True, 2)])
+def test_c1_fixture_first_steps_reproduce(fixture, w8a16, steps):
+    """Recompute prefill + the first decode steps of config 1 with the oracle (about 20 s per fixture) and
+    compare with the committed fixture: bf16 projections, and the weight-only int8 model."""
     import sys
     sys.path.insert(0, os.path.join(os.path.dirname(__file__), "golden"))
     import make_c1_golden as M
-    with open(os.path.join(os.path.dirname(__file__), "golden", "c1_greedy.json")) as f:
+    with open(os.path.join(os.path.dirname(__file__), "golden", fixture)) as f:
         gold = json.load(f)
     cfg = M.c1_config()
-    oracle = OracleQwen3(vars(cfg), M.c1_params(cfg))
-    ids, margins, topk = greedy_generate(oracle, M.c1_prompts(), max_tokens=3, block_size=256)
-    assert [r[:3] for r in gold["token_ids"]] == ids
-    for t in range(3):
+    oracle = OracleQwen3(vars(cfg), M.c1_params(cfg), w8a16=w8a16)
+    ids, margins, topk = greedy_generate(oracle, M.c1_prompts(), max_tokens=steps, block_size=256)
+    assert [r[:steps] for r in gold["token_ids"]] == ids
+    for t in range(steps):
         assert gold["top4_ids"][t] == topk[t][0]
         assert gold["top4_logits"][t] == topk[t][1]
+
+
+def test_w8a16_oracle_routes_the_projections_through_the_int8_linear():
+    """``w8a16=True``: every projection equals ``ops.w8a16_linear`` on ``ops.quantize_w8`` of its weight
+    (and differs from the bf16 product), embedding and LM head stay bf16; the quantised model is close
+    to the bf16 one (int8 per-channel error), not identical."""
+    params = tiny_params()
+    m8, m16 = OracleQwen3(TINY, params, w8a16=True), OracleQwen3(TINY, params)
+    name = "model.layers.1.mlp.down_proj.weight"
+    x = (torch.randn(5, params[name].shape[1], generator=torch.Generator().manual_seed(3))).to(torch.bfloat16)
+    wq, sc = O.quantize_w8(params[name])
+    assert torch.equal(m8.lin(x, name), O.w8a16_linear(x, wq, sc))
+    assert not torch.equal(m8.lin(x, name), m16.lin(x, name))
+    assert torch.equal(m8.lin(x[:, :TINY["hidden_size"]], "lm_head.weight"), m16.lin(x[:, :TINY["hidden_size"]], "lm_head.weight"))
+    assert set(m8.q8) == {k for k in params if k.endswith("proj.weight")}
+    prompts = [[3, 9, 27, 81, 243, 5, 6]]
+    _, _, t8 = greedy_generate(m8, prompts, max_tokens=1, block_size=8)
+    _, _, t16 = greedy_generate(m16, prompts, max_tokens=1, block_size=8)
+    a, b = torch.tensor(t8[0][1][0]), torch.tensor(t16[0][1][0])
+    assert (a - b).abs().max() < 0.25 * b.abs().max() and not torch.equal(a, b)
