@@ -207,6 +207,32 @@ int tlf_bf16_gemm(const void *x, int64_t x_stride, const void *w, void *y,
 int tlf_w8a16_gemm_silu_mul(const void *x, int64_t x_stride, const void *wq, const float *scale,
                             void *y, int32_t M, int32_t N, int32_t K, void *stream);
 
+/* Row-parallel projection fused with what follows it in a decoder layer: replaces
+ * RowParallelLinear.forward (layers/linear.py:181-183; o_proj, down_proj) followed by
+ * RMSNorm.add_rms_forward (layers/layernorm.py:33-45) of post_attention_layernorm, of the next
+ * layer's input_layernorm, or of the final norm (models/qwen3.py:163-166, 188-190).
+ *
+ *   h = bf16(scale[n] * sum_k x[m,k] wq[n,k])          (tlf_bf16_gemm_add_rmsnorm: no scale, w bf16)
+ *   s = h + residual (fp32);  residual_out = bf16(s)
+ *   y = bf16( bf16( s * rsqrt(mean(s^2) + eps) ) * norm_weight )
+ *
+ * residual, y, residual_out: bf16 [M, N] contiguous; norm_weight bf16 [N]; N <= 16384;
+ * residual_out may alias residual.  Bit-identical to the GEMM entry point followed by
+ * tlf_add_rmsnorm.  When the plan for (M, N, K) splits K across workgroups, the
+ * sum of the partial products, the residual add and the norm are one kernel (h never goes to
+ * memory); otherwise h is staged in the workspace and the two kernels run back to back.
+ * workspace: tlf_gemm_add_rmsnorm_workspace_bytes(M, N, K) bytes, 256-byte aligned.
+ * Other constraints as tlf_w8a16_gemm. */
+size_t tlf_gemm_add_rmsnorm_workspace_bytes(int32_t M, int32_t N, int32_t K);
+int tlf_w8a16_gemm_add_rmsnorm(const void *x, int64_t x_stride, const void *wq, const float *scale,
+                               const void *residual, const void *norm_weight, void *y,
+                               void *residual_out, int32_t M, int32_t N, int32_t K, float eps,
+                               void *workspace, size_t workspace_bytes, void *stream);
+int tlf_bf16_gemm_add_rmsnorm(const void *x, int64_t x_stride, const void *w, const void *residual,
+                              const void *norm_weight, void *y, void *residual_out, int32_t M,
+                              int32_t N, int32_t K, float eps, void *workspace,
+                              size_t workspace_bytes, void *stream);
+
 /* Diagnostic, no counterpart in the reference, touches no GPU: the kernel plan the two GEMM entry
  * points would use for a shape.  plan8 = {tile channels, tile tokens, LDS stages, waves/SIMD budget,
  * K-groups per workgroup, split-K factor, K per split, N-tile columns per XCD patch}; tile 0 x 0

@@ -155,12 +155,14 @@ def test_unfused_layer_path_gives_identical_tokens(llm_c1):
     runner = llm_c1.model_runner
     a = [o["token_ids"] for o in llm_c1.generate(prompts, sp)]
     runner.enforce_eager = True
+    runner.model.model.fused = False                  # the reference's op order: projection, then add-norm
     for layer in runner.model.model.layers:
-        layer.self_attn.fused = False
+        layer.self_attn.fused = False                 # q/k-norm, RoPE and KV store as separate kernels
     try:
         b = [o["token_ids"] for o in llm_c1.generate(prompts, sp)]
     finally:
         runner.enforce_eager = False
+        runner.model.model.fused = True
         for layer in runner.model.model.layers:
             layer.self_attn.fused = True
     assert a == b

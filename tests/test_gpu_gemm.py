@@ -116,3 +116,40 @@ def test_w8a16_gemm_fused_silu_mul_equals_the_two_kernels(M, N, K):
     ref = O.silu_and_mul(O.w8a16_linear(x, wq, scale))
     rel = ((fused.float().cpu() - ref.float()).norm() / ref.float().norm().clamp_min(1e-6)).item()
     assert rel <= 2e-3, rel
+
+
+@pytest.mark.parametrize("M,N,K,w8,path", [
+    (120, 4096, 4096, True, "fused"), (160, 4096, 12288, True, "fused"), (97, 1024, 3072, True, "fused"),
+    (120, 4096, 4096, False, "fused"), (70, 8704, 8192, True, "fused"), (50, 256, 8192, True, "fused"),
+    (40, 128, 4096, True, "fused"),
+    (256, 4096, 4096, True, "staged"), (4, 4096, 1024, True, "staged"), (2048, 1024, 3072, False, "staged")])
+def test_row_projection_with_add_rmsnorm_equals_the_two_kernels(M, N, K, w8, path):
+    """o_proj / down_proj together with the add-RMSNorm that follows: bit-identical to the GEMM entry point
+    followed by tlf_add_rmsnorm on both routes -- the fused split-K reduce + norm kernel ("fused", one case
+    per thread layout of the norm) and plans without a split ("staged")."""
+    import ctypes
+    from tinyllmforge_amd import _lib, ops as P
+    plan = (ctypes.c_int32 * 8)()
+    assert _lib.load().tlf_gemm_plan(M, N, K, int(w8), plan) == 0
+    assert (plan[5] > 1) == (path == "fused")
+    x = torch.randn(M, K, generator=g(M + 11)).to(BF)
+    res = torch.randn(M, N, generator=g(M + 12)).to(BF)
+    nw = (1 + 0.1 * torch.randn(N, generator=g(M + 13))).to(BF)
+    if w8:
+        w, scale = make_w8(N, K, N + 3)
+        scale = scale / 8                                   # outputs of the size of the residual
+        lin = P.w8a16_linear(x.to(DEV), w.to(DEV), scale.to(DEV))
+        ref_lin = O.w8a16_linear(x, w, scale)
+    else:
+        w, scale = (torch.randn(N, K, generator=g(N + 3)) / K ** 0.5).to(BF), None
+        lin = P.bf16_linear(x.to(DEV), w.to(DEV))
+        ref_lin = O.linear_exact(x, w)
+    y2, r2 = P.add_rms_norm(lin, res.to(DEV), nw.to(DEV), 1e-6)
+    y1, r1 = P.linear_add_rms_norm(x.to(DEV), w.to(DEV), None if scale is None else scale.to(DEV),
+                                   res.to(DEV), nw.to(DEV), 1e-6)
+    assert torch.equal(r1.view(torch.int16), r2.view(torch.int16))
+    assert torch.equal(y1.view(torch.int16), y2.view(torch.int16))
+    ref_y, ref_r = O.add_rms_norm(ref_lin, res, nw, 1e-6)
+    for got, ref in ((y1, ref_y), (r1, ref_r)):
+        rel = ((got.float().cpu() - ref.float()).norm() / ref.float().norm()).item()
+        assert rel <= 2e-3, rel

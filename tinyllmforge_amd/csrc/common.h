@@ -102,6 +102,63 @@ __device__ __forceinline__ void lds_barrier() {
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
 }
 
+// Second half of every RMSNorm kernel: TPR threads share a row, thread `sub` holds chunks
+// sub + c * TPR (8 values each) of s in v, of the norm weight in pw, and its own sum of squares in ss.
+//   n = bf16(s * rsqrt(mean(s^2) + eps));  y = bf16(float(n) * float(w))
+// (reference: tinyvllm/layers/layernorm.py:21-45).  The reduction tree is part of the result's bits,
+// which is why every kernel that ends in an RMSNorm shares this function and TLF_RMS_SHAPES.
+template <int TPR, int MAXC>
+__device__ __forceinline__ void rmsnorm_finish(const float (&v)[MAXC][8], const uint4 (&pw)[MAXC], float ss,
+                                               bool active, int sub, int nchunks, int cols, float eps,
+                                               unsigned short *__restrict__ y_row) {
+  if (TPR <= 64) {
+#pragma unroll
+    for (int o = TPR / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+  } else {
+    __shared__ float part[256 / 64];
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    ss = 0.f;
+#pragma unroll
+    for (int w = 0; w < TPR / 64; ++w) ss += part[w];
+  }
+  const float var = ss / static_cast<float>(cols);
+  const float inv = 1.0f / sqrtf(var + eps);
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int chunk = sub + c * TPR;
+    if (active && chunk < nchunks) {
+      float w[8];
+      unpack8(pw[c], w);
+      float o[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float n = bf16_bits_to_float(float_to_bf16_bits(__fmul_rn(v[c][i], inv)));
+        o[i] = __fmul_rn(n, w[i]);
+      }
+      *reinterpret_cast<uint4 *>(y_row + chunk * 8) = pack8(o);
+    }
+  }
+}
+
+// threads per row and chunks per thread for a row of `cols` values (256-thread workgroups,
+// 256 / TPR rows each); CALL(TPR, MAXC) is expanded for the matching shape
+#define TLF_RMS_SHAPES(cols, CALL) \
+  do {                             \
+    if ((cols) <= 128) {           \
+      CALL(16, 1);                 \
+    } else if ((cols) <= 512) {    \
+      CALL(64, 1);                 \
+    } else if ((cols) <= 2048) {   \
+      CALL(64, 4);                 \
+    } else if ((cols) <= 8192) {   \
+      CALL(256, 4);                \
+    } else {                       \
+      CALL(256, 8);                \
+    }                              \
+  } while (0)
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 inline int launch_status() {

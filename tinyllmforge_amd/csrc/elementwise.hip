@@ -49,36 +49,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(
       for (int i = 0; i < 8; ++i) ss = fmaf(v[c][i], v[c][i], ss);
     }
   }
-  // reduce over the TPR threads of the row
-  if (TPR <= 64) {
-#pragma unroll
-    for (int o = TPR / 2; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
-  } else {
-    __shared__ float part[256 / 64];
-    ss = wave_sum(ss);
-    if ((tid & 63) == 0) part[tid >> 6] = ss;
-    __syncthreads();
-    ss = 0.f;
-#pragma unroll
-    for (int w = 0; w < TPR / 64; ++w) ss += part[w];
-  }
-  const float var = ss / static_cast<float>(cols);
-  const float inv = 1.0f / sqrtf(var + eps);
-#pragma unroll
-  for (int c = 0; c < MAXC; ++c) {
-    const int chunk = sub + c * TPR;
-    if (active && chunk < nchunks) {
-      float w[8];
-      unpack8(pw[c], w);
-      float o[8];
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float n = bf16_bits_to_float(float_to_bf16_bits(__fmul_rn(v[c][i], inv)));
-        o[i] = __fmul_rn(n, w[i]);
-      }
-      *reinterpret_cast<uint4 *>(y + out_off + chunk * 8) = pack8(o);
-    }
-  }
+  rmsnorm_finish<TPR, MAXC>(v, pw, ss, active, sub, nchunks, cols, eps, y + out_off);
 }
 
 template <bool ADD>
@@ -95,11 +66,7 @@ int launch_rmsnorm(const void *x, int64_t x_outer_stride, const void *residual, 
                      dim3(static_cast<unsigned>((rows + (256 / TPR) - 1) / (256 / TPR))),         \
                      dim3(256), 0, stream, xs, x_outer_stride, rs, ws, ys, ro, rows, inner, cols, \
                      eps)
-  if (cols <= 128) TLF_RMS(16, 1);
-  else if (cols <= 512) TLF_RMS(64, 1);
-  else if (cols <= 2048) TLF_RMS(64, 4);
-  else if (cols <= 8192) TLF_RMS(256, 4);
-  else TLF_RMS(256, 8);
+  TLF_RMS_SHAPES(cols, TLF_RMS);
 #undef TLF_RMS
   return launch_status();
 }

@@ -473,6 +473,77 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmParams p) 
   *reinterpret_cast<uint2 *>(p.y + i4 * 4) = st;
 }
 
+// What follows a row-parallel projection in the decoder (o_proj, down_proj) is the residual add and
+// an RMSNorm (reference: tinyvllm/models/qwen3.py:163-166 after linear.py:181-183).  When K was
+// split across workgroups the projection's value only exists after the partial sums are added, so
+// this kernel is that sum and the add-RMSNorm in one pass:
+//   h = bf16(sum_k partial_k * scale)            -- exactly what splitk_reduce_kernel would store
+//   s = h + residual;  residual_out = bf16(s)
+//   y = bf16( bf16(s * rsqrt(mean(s^2) + eps)) * w )
+// Thread layout, summation order and rounding points are those of the stand-alone add-RMSNorm
+// kernel, so the two routes give the same bits.
+struct NormTail {
+  const unsigned short *residual;
+  const unsigned short *weight;
+  unsigned short *y;
+  unsigned short *residual_out;
+  float eps;
+};
+
+template <int TPR, int MAXC, bool W8>
+__global__ __launch_bounds__(256) void splitk_reduce_add_rmsnorm_kernel(const GemmParams p,
+                                                                        const NormTail t) {
+  constexpr int kRowsPerBlock = 256 / TPR;
+  const int tid = threadIdx.x;
+  const int sub = tid % TPR;
+  const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerBlock + tid / TPR;
+  const bool active = row < p.M;
+  const int nchunks = p.N / 8;
+  const int64_t mn = static_cast<int64_t>(p.M) * p.N;
+  const int64_t off = (active ? row : 0) * p.N;
+  float v[MAXC][8];
+  uint4 pw[MAXC];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int chunk = sub + c * TPR;
+    pw[c] = make_uint4(0, 0, 0, 0);
+    if (active && chunk < nchunks) {
+      pw[c] = *reinterpret_cast<const uint4 *>(t.weight + chunk * 8);
+      const uint4 pr = *reinterpret_cast<const uint4 *>(t.residual + off + chunk * 8);
+      const float *src = p.partial + off + chunk * 8;
+      float4 a = *reinterpret_cast<const float4 *>(src);
+      float4 b = *reinterpret_cast<const float4 *>(src + 4);
+      for (int k = 1; k < p.splits; ++k) {
+        const float4 a2 = *reinterpret_cast<const float4 *>(src + k * mn);
+        const float4 b2 = *reinterpret_cast<const float4 *>(src + k * mn + 4);
+        a.x += a2.x; a.y += a2.y; a.z += a2.z; a.w += a2.w;
+        b.x += b2.x; b.y += b2.y; b.z += b2.z; b.w += b2.w;
+      }
+      if (W8) {
+        const float4 s0 = *reinterpret_cast<const float4 *>(p.scale + chunk * 8);
+        const float4 s1 = *reinterpret_cast<const float4 *>(p.scale + chunk * 8 + 4);
+        a.x *= s0.x; a.y *= s0.y; a.z *= s0.z; a.w *= s0.w;
+        b.x *= s1.x; b.y *= s1.y; b.z *= s1.z; b.w *= s1.w;
+      }
+      uint4 hb;  // the projection's bf16 output
+      hb.x = pack_bf16x2(a.x, a.y);
+      hb.y = pack_bf16x2(a.z, a.w);
+      hb.z = pack_bf16x2(b.x, b.y);
+      hb.w = pack_bf16x2(b.z, b.w);
+      float r[8];
+      unpack8(hb, v[c]);
+      unpack8(pr, r);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[c][i] = __fadd_rn(v[c][i], r[i]);
+      *reinterpret_cast<uint4 *>(t.residual_out + off + chunk * 8) = pack8(v[c]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) ss = fmaf(v[c][i], v[c][i], ss);
+    }
+  }
+  rmsnorm_finish<TPR, MAXC>(v, pw, ss, active, sub, nchunks, p.N, t.eps, t.y + off);
+}
+
 // ---------------------------------------------------------------------------
 // Skinny GEMM for a handful of tokens (decode at small batch; up to 64 rows): weight-bandwidth bound.
 //
@@ -779,7 +850,8 @@ inline int skinny_max_m() {
 template <bool W8>
 int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *scale, void *y,
                 int32_t M, int32_t N, int32_t K, void *workspace, size_t workspace_bytes,
-                hipStream_t stream, int32_t *plan_out = nullptr, int32_t act = 0) {
+                hipStream_t stream, int32_t *plan_out = nullptr, int32_t act = 0,
+                const NormTail *tail = nullptr) {
   const bool dry = plan_out != nullptr;
   GemmParams p;
   p.x = static_cast<const unsigned char *>(x);
@@ -880,12 +952,48 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   int rc = launch_status();
   if (rc != TLF_OK) return rc;
   if (g.splits > 1) {
+    if (tail) {  // the caller checked that this plan splits K and that the row fits the kernel
+#define TLF_TAIL(TPR_, MAXC_)                                                                 \
+  hipLaunchKernelGGL((splitk_reduce_add_rmsnorm_kernel<TPR_, MAXC_, W8>),                     \
+                     dim3(static_cast<unsigned>((M + (256 / TPR_) - 1) / (256 / TPR_))), dim3(256), 0, \
+                     stream, p, *tail)
+      TLF_RMS_SHAPES(N, TLF_TAIL);
+#undef TLF_TAIL
+      return launch_status();
+    }
     const int64_t total4 = static_cast<int64_t>(M) * N / 4;
     hipLaunchKernelGGL((splitk_reduce_kernel<W8>), dim3(static_cast<unsigned>((total4 + 255) / 256)),
                        dim3(256), 0, stream, p);
     rc = launch_status();
   }
   return rc;
+}
+
+inline size_t align256(size_t n) { return (n + 255) & ~static_cast<size_t>(255); }
+
+// Projection followed by add-RMSNorm.  A plan that splits K across workgroups ends in the fused
+// reduce + norm kernel; every other plan writes the projection to the head of the workspace and
+// runs the stand-alone add-RMSNorm on it.
+template <bool W8>
+int launch_gemm_add_rmsnorm(const void *x, int64_t x_stride, const void *w, const float *scale,
+                            const NormTail &tail, int32_t M, int32_t N, int32_t K, void *workspace,
+                            size_t workspace_bytes, hipStream_t stream) {
+  int32_t plan[8];
+  int rc = launch_gemm<W8>(nullptr, K, nullptr, nullptr, nullptr, M, N, K, nullptr, 0, nullptr, plan);
+  if (rc != TLF_OK) return rc;
+  const bool fused = plan[5] > 1;
+  if (fused)
+    return launch_gemm<W8>(x, x_stride, w, scale, nullptr, M, N, K, workspace, workspace_bytes, stream,
+                           nullptr, 0, &tail);
+  const size_t tmp_bytes = align256(static_cast<size_t>(M) * N * 2);
+  if (!workspace || workspace_bytes < tmp_bytes || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+    return TLF_E_WORKSPACE;
+  unsigned char *ws = static_cast<unsigned char *>(workspace);
+  rc = launch_gemm<W8>(x, x_stride, w, scale, ws, M, N, K, ws + tmp_bytes, workspace_bytes - tmp_bytes,
+                       stream);
+  if (rc != TLF_OK) return rc;
+  return tlf_add_rmsnorm(ws, tail.residual, tail.weight, tail.y, tail.residual_out, M, N, tail.eps,
+                         stream);
 }
 
 inline int check_gemm_args(const void *x, int64_t x_stride, const void *w, const void *y, int32_t M,
@@ -946,4 +1054,53 @@ extern "C" int tlf_w8a16_gemm_silu_mul(const void *x, int64_t x_stride, const vo
   if (reinterpret_cast<uintptr_t>(scale) & 15u) return TLF_E_ALIGN;
   return launch_gemm<true>(x, x_stride, wq, scale, y, M, N, K, nullptr, 0,
                            static_cast<hipStream_t>(stream), nullptr, 1);
+}
+
+extern "C" size_t tlf_gemm_add_rmsnorm_workspace_bytes(int32_t M, int32_t N, int32_t K) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % kBK) return 0;
+  return align256(static_cast<size_t>(M) * N * 2) + align256(tlf_w8a16_gemm_workspace_bytes(M, N, K));
+}
+
+static int check_norm_tail(const void *residual, const void *norm_weight, const void *y,
+                           const void *residual_out, int32_t N) {
+  if (!residual || !norm_weight || !y || !residual_out) return TLF_E_NULL;
+  if (N > 16384) return TLF_E_SHAPE;
+  if (!aligned16(residual) || !aligned16(norm_weight) || !aligned16(y) || !aligned16(residual_out))
+    return TLF_E_ALIGN;
+  return TLF_OK;
+}
+
+extern "C" int tlf_w8a16_gemm_add_rmsnorm(const void *x, int64_t x_stride, const void *wq,
+                                          const float *scale, const void *residual,
+                                          const void *norm_weight, void *y, void *residual_out,
+                                          int32_t M, int32_t N, int32_t K, float eps,
+                                          void *workspace, size_t workspace_bytes, void *stream) {
+  if (M == 0) return TLF_OK;
+  int rc = check_gemm_args(x, x_stride, wq, y, M, N, K);
+  if (rc != TLF_OK) return rc;
+  if (!scale) return TLF_E_NULL;
+  if (reinterpret_cast<uintptr_t>(scale) & 15u) return TLF_E_ALIGN;
+  rc = check_norm_tail(residual, norm_weight, y, residual_out, N);
+  if (rc != TLF_OK) return rc;
+  const NormTail tail{static_cast<const unsigned short *>(residual),
+                      static_cast<const unsigned short *>(norm_weight),
+                      static_cast<unsigned short *>(y), static_cast<unsigned short *>(residual_out), eps};
+  return launch_gemm_add_rmsnorm<true>(x, x_stride, wq, scale, tail, M, N, K, workspace, workspace_bytes,
+                                       static_cast<hipStream_t>(stream));
+}
+
+extern "C" int tlf_bf16_gemm_add_rmsnorm(const void *x, int64_t x_stride, const void *w,
+                                         const void *residual, const void *norm_weight, void *y,
+                                         void *residual_out, int32_t M, int32_t N, int32_t K, float eps,
+                                         void *workspace, size_t workspace_bytes, void *stream) {
+  if (M == 0) return TLF_OK;
+  int rc = check_gemm_args(x, x_stride, w, y, M, N, K);
+  if (rc != TLF_OK) return rc;
+  rc = check_norm_tail(residual, norm_weight, y, residual_out, N);
+  if (rc != TLF_OK) return rc;
+  const NormTail tail{static_cast<const unsigned short *>(residual),
+                      static_cast<const unsigned short *>(norm_weight),
+                      static_cast<unsigned short *>(y), static_cast<unsigned short *>(residual_out), eps};
+  return launch_gemm_add_rmsnorm<false>(x, x_stride, w, nullptr, tail, M, N, K, workspace, workspace_bytes,
+                                        static_cast<hipStream_t>(stream));
 }

@@ -144,6 +144,15 @@ class RowParallelLinear(LinearBase):
         self.input_size_per_partition = input_size // self.tp_size
         self._make_params(output_size, self.input_size_per_partition, bias)
 
+    def forward_add_rmsnorm(self, x: torch.Tensor, residual: torch.Tensor, norm):
+        """``norm(self(x), residual)`` (layernorm.py:33-45 after linear.py:181-183) behind one call;
+        ``norm`` is the ``RMSNorm`` module that follows this projection.  Returns ``(normed, residual)``."""
+        if self.bias is not None:
+            return norm(self.forward(x), residual)
+        if self.qweight is not None:
+            return ops.linear_add_rms_norm(x, self.qweight, self.qscale, residual, norm.weight.data, norm.eps)
+        return ops.linear_add_rms_norm(x, self.weight.data, None, residual, norm.weight.data, norm.eps)
+
     def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor):
         n = param.data.size(self.tp_dim)
         param.data.copy_(loaded_weight.narrow(self.tp_dim, self.tp_rank * n, n))

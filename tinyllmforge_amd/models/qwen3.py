@@ -1,8 +1,9 @@
 """Qwen3 decoder wiring (reference: tinyvllm/models/qwen3.py:14-234), one GPU.
 
 Same module tree, parameter names and op order as the reference.  With ``fused=True`` (default)
-the q/k-norm, RoPE and KV-cache store of a layer run as one kernel; every rounding of the
-unfused sequence is kept, so both paths give identical bits.
+the q/k-norm, RoPE and KV-cache store of a layer run as one kernel, and each row-parallel
+projection (o_proj, down_proj) runs together with the add-RMSNorm that consumes it; every
+rounding of the unfused sequence is kept, so both paths give identical bits.
 """
 import torch
 from torch import nn
@@ -37,7 +38,9 @@ class QWen3Attention(nn.Module):
         self.q_norm = RMSNorm(self.head_dim, eps=rms_norm_eps)
         self.k_norm = RMSNorm(self.head_dim, eps=rms_norm_eps)
 
-    def forward(self, positions: torch.Tensor, hidden_states: torch.Tensor) -> torch.Tensor:
+    def forward(self, positions: torch.Tensor, hidden_states: torch.Tensor, residual=None, norm=None):
+        """``o_proj(attention(...))``; with ``norm`` (the RMSNorm that follows, and its ``residual``) the
+        projection and the add-norm are one call and ``(normed, residual)`` is returned."""
         qkv = self.qkv_proj(hidden_states)
         if self.fused:
             ctx = get_context()
@@ -57,6 +60,8 @@ class QWen3Attention(nn.Module):
             k = self.k_norm(k.view(-1, self.num_kv_heads, self.head_dim)).view(-1, self.kv_size)
             q, k = self.rotary_emb(positions, q, k)
             o = self.attn(q, k, v)
+        if norm is not None:
+            return self.o_proj.forward_add_rmsnorm(o, residual, norm)
         return self.o_proj(o)
 
 
@@ -68,9 +73,12 @@ class Qwen3MLP(nn.Module):
         self.down_proj = RowParallelLinear(intermediate_size, hidden_size, bias=False)
         self.act_fn = SiluAndMul()
 
-    def forward(self, x: torch.Tensor) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, residual=None, norm=None):
         # gate_up projection and activation in one kernel when the weights are int8 (qwen3.py:123-130)
-        return self.down_proj(self.gate_up_proj.forward_silu_mul(x))
+        act = self.gate_up_proj.forward_silu_mul(x)
+        if norm is not None:   # down_proj together with the add-norm that follows the layer
+            return self.down_proj.forward_add_rmsnorm(act, residual, norm)
+        return self.down_proj(act)
 
 
 class Qwen3DecoderLayer(nn.Module):
@@ -84,6 +92,14 @@ class Qwen3DecoderLayer(nn.Module):
         self.mlp = Qwen3MLP(config.hidden_size, config.intermediate_size, config.hidden_act)
         self.input_layernorm = RMSNorm(config.hidden_size, eps=config.rms_norm_eps)
         self.post_attention_layernorm = RMSNorm(config.hidden_size, eps=config.rms_norm_eps)
+        self.fused = fused
+
+    def forward_normed(self, positions, normed, residual, next_norm):
+        """The layer from after its input norm to after the NEXT norm (the following layer's
+        ``input_layernorm`` or the model's final norm): each row-parallel projection runs together with
+        the add-norm that consumes it.  Same ops and rounding points as ``forward`` chained with that norm."""
+        hidden_states, residual = self.self_attn(positions, normed, residual, self.post_attention_layernorm)
+        return self.mlp(hidden_states, residual, next_norm)
 
     def forward(self, positions, hidden_states, residual):
         if residual is None:                                   # first layer: the embedding is the residual
@@ -103,9 +119,17 @@ class Qwen3Model(nn.Module):
         self.embed_tokens = VocabParallelEmbedding(config.vocab_size, config.hidden_size)
         self.layers = nn.ModuleList([Qwen3DecoderLayer(config, fused) for _ in range(config.num_hidden_layers)])
         self.norm = RMSNorm(config.hidden_size, config.rms_norm_eps)
+        self.fused = fused
 
     def forward(self, input_ids: torch.Tensor, positions: torch.Tensor) -> torch.Tensor:
         hidden_states = self.embed_tokens(input_ids)
+        if self.fused:
+            residual = hidden_states                      # the embedding is the first residual
+            hidden_states = self.layers[0].input_layernorm(hidden_states)
+            for i, layer in enumerate(self.layers):
+                nxt = self.layers[i + 1].input_layernorm if i + 1 < len(self.layers) else self.norm
+                hidden_states, residual = layer.forward_normed(positions, hidden_states, residual, nxt)
+            return hidden_states
         residual = None
         for layer in self.layers:
             hidden_states, residual = layer(positions, hidden_states, residual)

@@ -249,6 +249,36 @@ def bf16_linear(x, w):
     return y.view(*x.shape[:-1], N)
 
 
+def linear_add_rms_norm(x, w, scale, residual, norm_weight, eps):
+    """``add_rms_norm(linear(x), residual)`` behind one call: ``w`` int8 with ``scale`` (weight-only int8)
+    or bf16 with ``scale=None``.  Returns ``(normed, new_residual)``, the bits of the two separate calls."""
+    lib = _lib.load()
+    w8 = scale is not None
+    _need(x, BF16, "x"); _need(w, torch.int8 if w8 else BF16, "w")
+    _need(residual, BF16, "residual"); _need(norm_weight, BF16, "norm_weight")
+    assert x.stride(-1) == 1 and w.is_contiguous() and residual.is_contiguous()
+    x2 = x.reshape(-1, x.shape[-1])
+    M, K = x2.shape
+    N = w.shape[0]
+    assert residual.numel() == M * N
+    y = torch.empty(M, N, dtype=BF16, device=x.device)
+    r = torch.empty(M, N, dtype=BF16, device=x.device)
+    ws = _workspace(lib.tlf_gemm_add_rmsnorm_workspace_bytes(M, N, K), x.device, "gemm")
+    if w8:
+        _need(scale, torch.float32, "scale")
+        check(lib.tlf_w8a16_gemm_add_rmsnorm(
+            x2.data_ptr(), x2.stride(0), w.data_ptr(), scale.data_ptr(), residual.data_ptr(),
+            norm_weight.data_ptr(), y.data_ptr(), r.data_ptr(), M, N, K, float(eps), ws.data_ptr(),
+            ws.numel(), _stream()), "tlf_w8a16_gemm_add_rmsnorm")
+    else:
+        check(lib.tlf_bf16_gemm_add_rmsnorm(
+            x2.data_ptr(), x2.stride(0), w.data_ptr(), residual.data_ptr(), norm_weight.data_ptr(),
+            y.data_ptr(), r.data_ptr(), M, N, K, float(eps), ws.data_ptr(), ws.numel(), _stream()),
+            "tlf_bf16_gemm_add_rmsnorm")
+    shape = (*x.shape[:-1], N)
+    return y.view(shape), r.view(shape)
+
+
 # ------------------------------------------------------------------ a3
 def paged_decode_attention(q, k_cache, v_cache, context_lens, block_tables, scale,
                            k_scale=None, v_scale=None):
