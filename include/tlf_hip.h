@@ -233,6 +233,22 @@ int tlf_bf16_gemm_add_rmsnorm(const void *x, int64_t x_stride, const void *w, co
                               int32_t N, int32_t K, float eps, void *workspace,
                               size_t workspace_bytes, void *stream);
 
+/* LM head fused with the greedy sample: replaces ParallelLMHead.forward's product
+ * (layers/embed_head.py:63) followed by Sampler.forward's greedy branch (layers/sampler.py:13-14,21)
+ * when every temperature of the batch is 0.
+ *
+ *   token_ids[m] = argmax_n bf16( sum_k x[m,k] * w[n,k] ),  first index among ties      int64 [M]
+ *
+ * The [M, N] logits are never stored (more than 16 tokens; a smaller batch stages them in the
+ * workspace): the GEMM epilogue keeps one (value, index) key per token, N-tile and wave, and a
+ * second small kernel takes their maximum.  Identical to tlf_bf16_gemm followed by tlf_argmax.
+ * workspace: tlf_gemm_argmax_workspace_bytes(M, N, K) bytes, 256-byte aligned.
+ * Other constraints as tlf_bf16_gemm. */
+size_t tlf_gemm_argmax_workspace_bytes(int32_t M, int32_t N, int32_t K);
+int tlf_bf16_gemm_argmax(const void *x, int64_t x_stride, const void *w, int64_t *token_ids,
+                         int32_t M, int32_t N, int32_t K,
+                         void *workspace, size_t workspace_bytes, void *stream);
+
 /* Diagnostic, no counterpart in the reference, touches no GPU: the kernel plan the two GEMM entry
  * points would use for a shape.  plan8 = {tile channels, tile tokens, LDS stages, waves/SIMD budget,
  * K-groups per workgroup, split-K factor, K per split, N-tile columns per XCD patch}; tile 0 x 0

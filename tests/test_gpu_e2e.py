@@ -148,6 +148,23 @@ def test_c1_eager_equals_graph_and_rerun_hits_prefix_cache(llm_c1, golden):
     assert a == b
 
 
+def test_fused_lm_head_argmax_gives_the_tokens_of_logits_then_sampler(llm_c1):
+    """All-greedy batches sample through the fused LM head + argmax; with it switched off the same batch goes
+    through logits and the sampler kernel.  Same tokens, prefill (4 last rows) and graph decode alike."""
+    from tinyllmforge_amd import SamplingParams
+    sp = SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True)
+    prompts = [p[:50 + 7 * i] for i, p in enumerate(c1_prompts())]
+    runner = llm_c1.model_runner
+    assert runner.fused_greedy
+    a = [o["token_ids"] for o in llm_c1.generate(prompts, sp)]
+    runner.fused_greedy = False
+    try:
+        b = [o["token_ids"] for o in llm_c1.generate(prompts, sp)]
+    finally:
+        runner.fused_greedy = True
+    assert a == b
+
+
 def test_unfused_layer_path_gives_identical_tokens(llm_c1):
     from tinyllmforge_amd import SamplingParams
     sp = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)

@@ -153,3 +153,27 @@ def test_row_projection_with_add_rmsnorm_equals_the_two_kernels(M, N, K, w8, pat
     for got, ref in ((y1, ref_y), (r1, ref_r)):
         rel = ((got.float().cpu() - ref.float()).norm() / ref.float().norm()).item()
         assert rel <= 2e-3, rel
+
+
+@pytest.mark.parametrize("M,N,K", [(4, 4112, 256), (40, 4112, 512), (130, 9008, 256), (300, 20000, 128), (256, 151936, 64)])
+def test_lm_head_with_greedy_sample_equals_gemm_then_argmax(M, N, K):
+    """LM head + argmax in one call (no logits stored) against the two entry points it replaces, on logits
+    full of exact ties: the vocabulary rows are drawn from 61 distinct vectors, so every value -- the
+    maximum included -- occurs many times and the FIRST index must win (sampler.py:21, torch.argmax)."""
+    from tinyllmforge_amd import ops as P
+    base = (torch.randn(61, K, generator=g(N)) / K ** 0.5).to(BF)
+    which = torch.randint(0, 61, (N,), generator=g(N + 1))
+    w = base[which].contiguous()
+    x = torch.randn(M, K, generator=g(M + 5)).to(BF)
+    ids = P.bf16_linear_argmax(x.to(DEV), w.to(DEV))
+    assert ids.dtype == torch.int64 and ids.shape == (M,)
+    logits = P.bf16_linear(x.to(DEV), w.to(DEV))
+    two = P.argmax(logits)
+    assert torch.equal(ids, two) and torch.equal(ids, logits.float().argmax(-1))
+    ids = ids.cpu()
+    first = torch.full((61,), N, dtype=torch.int64).scatter_reduce(0, which, torch.arange(N), "amin")
+    assert torch.equal(ids, first[which[ids]])                       # first index of its tie group
+    ref = O.linear_exact(x, base).float()                             # [M, 61] oracle logits per distinct row
+    top = ref.max(-1).values
+    got = ref.gather(1, which[ids][:, None])[:, 0]
+    assert ((top - got) <= O.bf16_ulp(top)).all()                      # and that group is the oracle's maximum

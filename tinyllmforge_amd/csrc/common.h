@@ -159,6 +159,29 @@ __device__ __forceinline__ void rmsnorm_finish(const float (&v)[MAXC][8], const 
     }                              \
   } while (0)
 
+// Greedy argmax (reference: tinyvllm/layers/sampler.py:13-14,21) as a maximum over 64-bit keys:
+// key = (order-preserving image of the bf16 value) << 32 | (~index), so the largest key is the
+// largest value with the smallest index among ties.  Key 0 is below every real key.
+__device__ __forceinline__ unsigned long long argmax_key(unsigned short bits, unsigned int idx) {
+  if (bits == 0x8000u) bits = 0;  // -0 == +0
+  const unsigned int ord = (bits & 0x8000u) ? (~bits & 0xffffu) : (bits | 0x8000u);
+  return (static_cast<unsigned long long>(ord) << 32) | (0xffffffffu - idx);
+}
+
+__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    unsigned int lo = __shfl_xor(static_cast<unsigned int>(v), o, 64);
+    unsigned int hi = __shfl_xor(static_cast<unsigned int>(v >> 32), o, 64);
+    unsigned long long other = (static_cast<unsigned long long>(hi) << 32) | lo;
+    v = other > v ? other : v;
+  }
+  return v;
+}
+
+int launch_argmax_final(const unsigned long long *keys, int32_t nparts, int64_t *out, int32_t rows,
+                        hipStream_t stream);
+
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 inline int launch_status() {

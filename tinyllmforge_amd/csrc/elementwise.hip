@@ -251,23 +251,6 @@ __global__ __launch_bounds__(256) void embedding_kernel(const int64_t *__restric
 // key is the largest value with the smallest index among ties.
 constexpr int kArgmaxMaxChunks = 128;
 
-__device__ __forceinline__ unsigned long long argmax_key(unsigned short bits, unsigned int idx) {
-  if (bits == 0x8000u) bits = 0;  // -0 == +0
-  const unsigned int ord = (bits & 0x8000u) ? (~bits & 0xffffu) : (bits | 0x8000u);
-  return (static_cast<unsigned long long>(ord) << 32) | (0xffffffffu - idx);
-}
-
-__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) {
-    unsigned int lo = __shfl_xor(static_cast<unsigned int>(v), o, 64);
-    unsigned int hi = __shfl_xor(static_cast<unsigned int>(v >> 32), o, 64);
-    unsigned long long other = (static_cast<unsigned long long>(hi) << 32) | lo;
-    v = other > v ? other : v;
-  }
-  return v;
-}
-
 __global__ __launch_bounds__(256) void argmax_partial_kernel(
     const unsigned short *__restrict__ logits, int64_t row_stride, int32_t vocab,
     unsigned long long *__restrict__ partial, int32_t nchunks) {
@@ -315,6 +298,13 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(
   }
   best = wave_max_u64(best);
   if (threadIdx.x == 0) out[row] = static_cast<int64_t>(0xffffffffu - static_cast<unsigned int>(best));
+}
+
+// Last stage of the greedy sample on its own: rows x nparts keys (argmax_key) -> token ids.
+int launch_argmax_final(const unsigned long long *keys, int32_t nparts, int64_t *out, int32_t rows,
+                        hipStream_t stream) {
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(64), 0, stream, keys, nparts, out);
+  return launch_status();
 }
 
 inline int argmax_chunks(int32_t rows, int32_t vocab) {

@@ -49,6 +49,9 @@ struct GemmParams {
   int32_t m_tiles, n_tiles;
   int32_t group_n;  // N-tile columns walked together by one XCD
   int32_t act;      // 1: SiLU-and-mul epilogue over interleaved gate/up channels, y is [M, N/2]
+                    // 2: greedy-sample epilogue, nothing but argmax keys [M, amax_parts] is stored
+  unsigned long long *amax;
+  int32_t amax_parts;  // key columns per token: one per (N-tile, wave along N)
 };
 
 // Epilogue of the tiled kernel (BN output channels x BM tokens per workgroup, waves laid out as
@@ -59,13 +62,50 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
                                               int n0, int wn, int wm, int r, int kg, int split) {
   // Epilogue.  acc[i][j][v]: token m = m0 + wm*WM + j*32 + r,
   // channel n = n0 + wn*WN + i*32 + (v/4)*8 + kg*4 + (v%4).
+  if (p.act == 2) {
+    // LM head + greedy sample (reference: tinyvllm/layers/embed_head.py:63, sampler.py:13-14,21): the
+    // logits are never stored.  A token's channels of this wave sit in the registers of lanes r and
+    // r + 32: each lane keeps the best key of its bf16-rounded values, the pair is merged with one
+    // exchange, and the key goes to column (N-tile, wave) of the token's row.
+    const int part = (n0 + wn * WN) / WN;
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      const int m = m0 + wm * WM + j * 32 + r;
+      unsigned long long best = 0;
+#pragma unroll
+      for (int i = 0; i < TN; ++i)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = n0 + wn * WN + i * 32 + q * 8 + kg * 4;
+          if (n >= p.N) continue;
+          float o[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) o[e] = acc[i][j][q * 4 + e];
+          if (W8) {
+            const float4 s = *reinterpret_cast<const float4 *>(p.scale + n);
+            o[0] *= s.x; o[1] *= s.y; o[2] *= s.z; o[3] *= s.w;
+          }
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const unsigned long long key = argmax_key(float_to_bf16_bits(o[e]), static_cast<unsigned int>(n + e));
+            best = key > best ? key : best;
+          }
+        }
+      const unsigned int lo = __shfl_xor(static_cast<unsigned int>(best), 32, 64);
+      const unsigned int hi = __shfl_xor(static_cast<unsigned int>(best >> 32), 32, 64);
+      const unsigned long long other = (static_cast<unsigned long long>(hi) << 32) | lo;
+      best = other > best ? other : best;
+      if (kg == 0 && m < p.M) p.amax[static_cast<int64_t>(m) * p.amax_parts + part] = best;
+    }
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < TM; ++j) {
     const int m = m0 + wm * WM + j * 32 + r;
     if (m >= p.M) continue;
 #pragma unroll
     for (int i = 0; i < TN; ++i) {
-      if (p.act) {
+      if (p.act == 1) {
         // channels come in groups of 16 = 8 gate rows then the 8 matching up rows, so this lane's
         // registers q = 0, 2 hold gate values and q = 1, 3 the up values of the same 4 channels
 #pragma unroll
@@ -788,6 +828,10 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
       // (measured 42.6 -> 38.2 us at M = 130, 55.7 -> 44.5 us at M = 256 on 4096 x 12288)
       g.bn = 128; g.bm = 64; g.stages = 4; g.occ = 3;
       splits = 4;
+      if (M > 160) {
+        // two M-tiles of 128 with cold weights: 43.3 -> 41.2 us at M = 192, 46.4 -> 40.7 us at M = 256
+        g.bm = 128; g.stages = 3; g.occ = 2; g.wn = 2;
+      }
     }
   } else if (tiles(128, 128) < 256) {
     g.bn = 128; g.bm = 64; g.stages = 2; g.occ = 3;
@@ -862,6 +906,8 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   p.partial = nullptr;
   p.M = M; p.N = N; p.K = K;
   p.act = act;
+  p.amax = nullptr;
+  p.amax_parts = 0;
   if (M <= skinny_max_m()) {
     p.k_per_split = K; p.splits = 1; p.m_tiles = 1; p.n_tiles = 1; p.group_n = 1;
     if (dry) {
@@ -869,6 +915,7 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
       for (int i = 0; i < 8; ++i) plan_out[i] = skinny[i];
       return TLF_OK;
     }
+    if (act == 2) return TLF_E_UNSUPPORTED;  // the caller stages the logits and runs tlf_argmax
     return launch_skinny<W8>(p, stream);
   }
   GemmPlan g = plan_gemm(M, N, K, W8);
@@ -890,6 +937,12 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   p.splits = g.splits;
   p.m_tiles = (M + g.bm - 1) / g.bm;
   p.n_tiles = (N + g.bn - 1) / g.bn;
+  if (act == 2 && !dry) {  // argmax keys: at most N / 32 + 8 columns per token for any tile shape
+    const size_t need = static_cast<size_t>(M) * (N / 32 + 8) * sizeof(unsigned long long);
+    if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15u))
+      return TLF_E_WORKSPACE;
+    p.amax = static_cast<unsigned long long *>(workspace);
+  }
   if (g.splits > 1 && !dry) {
     const size_t need = static_cast<size_t>(g.splits) * M * N * sizeof(float);
     if (!workspace || workspace_bytes < need || (reinterpret_cast<uintptr_t>(workspace) & 15u))
@@ -910,6 +963,7 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
 #define TLF_TILE_KG(BN_, BM_, WN_, WM_, NS_, OCC_, KG_)                                     \
   if (!launched && g.bn == BN_ && g.bm == BM_ && g.stages == NS_ && g.occ == OCC_ &&        \
       g.kgroups == KG_ && (g.wn == 0 || g.wn == WN_)) {                                                                   \
+    p.amax_parts = p.n_tiles * WN_;                                                         \
     if (!dry)                                                                               \
       hipLaunchKernelGGL((gemm_dlds_kernel<BN_, BM_, WN_, WM_, W8, NS_, OCC_, KG_>), grid,  \
                          dim3(WN_ * WM_ * KG_ * 64), 0, stream, p);                         \
@@ -951,6 +1005,8 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   if (!launched) return TLF_E_UNSUPPORTED;
   int rc = launch_status();
   if (rc != TLF_OK) return rc;
+  if (act == 2)  // y is the int64 token-id vector here
+    return launch_argmax_final(p.amax, p.amax_parts, static_cast<int64_t *>(y), M, stream);
   if (g.splits > 1) {
     if (tail) {  // the caller checked that this plan splits K and that the row fits the kernel
 #define TLF_TAIL(TPR_, MAXC_)                                                                 \
@@ -1103,4 +1159,34 @@ extern "C" int tlf_bf16_gemm_add_rmsnorm(const void *x, int64_t x_stride, const 
                       static_cast<unsigned short *>(y), static_cast<unsigned short *>(residual_out), eps};
   return launch_gemm_add_rmsnorm<false>(x, x_stride, w, nullptr, tail, M, N, K, workspace, workspace_bytes,
                                         static_cast<hipStream_t>(stream));
+}
+
+// LM head + greedy sample.  Tiled plans never store the logits; for a handful of tokens (skinny
+// kernel) they are staged in the workspace and tlf_argmax runs on them.
+extern "C" size_t tlf_gemm_argmax_workspace_bytes(int32_t M, int32_t N, int32_t K) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % kBK) return 0;
+  const size_t keys = align256(static_cast<size_t>(M) * (N / 32 + 8) * sizeof(unsigned long long));
+  const size_t staged = align256(static_cast<size_t>(M) * N * 2) + align256(tlf_argmax_workspace_bytes(M, N));
+  return keys > staged ? keys : staged;
+}
+
+extern "C" int tlf_bf16_gemm_argmax(const void *x, int64_t x_stride, const void *w, int64_t *token_ids,
+                                    int32_t M, int32_t N, int32_t K, void *workspace,
+                                    size_t workspace_bytes, void *stream) {
+  if (M == 0) return TLF_OK;
+  int rc = check_gemm_args(x, x_stride, w, token_ids, M, N, K);
+  if (rc != TLF_OK) return rc;
+  if (!workspace || workspace_bytes < tlf_gemm_argmax_workspace_bytes(M, N, K) ||
+      (reinterpret_cast<uintptr_t>(workspace) & 255u))
+    return TLF_E_WORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (M <= skinny_max_m()) {
+    unsigned char *ws = static_cast<unsigned char *>(workspace);
+    const size_t tmp = align256(static_cast<size_t>(M) * N * 2);
+    rc = launch_gemm<false>(x, x_stride, w, nullptr, ws, M, N, K, nullptr, 0, st);
+    if (rc != TLF_OK) return rc;
+    return tlf_argmax(ws, N, token_ids, M, N, ws + tmp, workspace_bytes - tmp, stream);
+  }
+  return launch_gemm<false>(x, x_stride, w, nullptr, token_ids, M, N, K, workspace, workspace_bytes, st,
+                            nullptr, 2);
 }

@@ -54,6 +54,7 @@ class ModelRunner:
             torch.set_default_dtype(default_dtype)
         self.model.eval()
         self.sampler = Sampler()
+        self.fused_greedy = True      # all-greedy batches: LM head and argmax in one call
         self.graphs = {}
         self.graph_bs = []
         with torch.inference_mode():
@@ -155,10 +156,11 @@ class ModelRunner:
 
     # ------------------------------------------------------------------ forward
     @torch.inference_mode()
-    def run_model(self, input_ids, positions, is_prefill):
+    def run_hidden(self, input_ids, positions, is_prefill):
+        """Final hidden states of the step's tokens (eager, or a graph replay with device-side inputs)."""
         bs = input_ids.size(0)
         if is_prefill or self.enforce_eager or not self.graph_bs or bs > self.graph_bs[-1]:
-            return self.model.compute_logits(self.model(input_ids, positions))
+            return self.model(input_ids, positions)
         ctx = get_context()
         gbs = next(x for x in self.graph_bs if x >= bs)
         gv = self.graph_vars
@@ -174,13 +176,18 @@ class ModelRunner:
         w = ctx.block_tables.size(1)
         gv["block_tables"][:bs, :w] = ctx.block_tables
         self.graphs[gbs].replay()
-        return self.model.compute_logits(gv["outputs"][:bs])
+        return gv["outputs"][:bs]
+
+    @torch.inference_mode()
+    def run_model(self, input_ids, positions, is_prefill):
+        return self.model.compute_logits(self.run_hidden(input_ids, positions, is_prefill))
 
     @torch.inference_mode()
     def run_decode_graph(self, seqs):
         """Decode step through a captured graph: the integer inputs (I.decode_inputs, the same function the
         eager path uploads) are written straight into the pinned mirror of the graph's static buffers,
-        padding rows get slot -1 (no cache write) and length 0 (no cache read), one H2D copy, replay."""
+        padding rows get slot -1 (no cache write) and length 0 (no cache read), one H2D copy, replay.
+        Returns the final hidden states."""
         bs = len(seqs)
         gbs = next(x for x in self.graph_bs if x >= bs)
         d = I.decode_inputs(seqs, self.block_size, self.config.decode_position_quirk)
@@ -199,7 +206,16 @@ class ModelRunner:
         self.graph_pack_dev.copy_(self.graph_pack_host, non_blocking=True)
         set_context(False)
         self.graphs[gbs].replay()
-        return self.model.compute_logits(self.graph_vars["outputs"][:bs])
+        return self.graph_vars["outputs"][:bs]
+
+    @torch.inference_mode()
+    def sample(self, hidden, temperatures):
+        """Token ids from the final hidden states.  An all-greedy batch goes through the fused LM head +
+        argmax (no logits in memory); otherwise logits, then the sampler.  The ``tolist`` is the step's one
+        device sync."""
+        if self._all_greedy and self.fused_greedy:
+            return self.model.compute_greedy_ids(hidden).tolist()
+        return self.sampler(self.model.compute_logits(hidden), temperatures, self._all_greedy).tolist()
 
     def run(self, seqs, is_prefill):
         use_graph = (not is_prefill and not self.enforce_eager and self.graph_bs
@@ -207,14 +223,12 @@ class ModelRunner:
                      and max(len(s.block_table) for s in seqs) <= self.graph_max_blocks)
         if use_graph:
             temperatures = self.prepare_sample(seqs)
-            logits = self.run_decode_graph(seqs)
-            token_ids = self.sampler(logits, temperatures, self._all_greedy).tolist()
+            token_ids = self.sample(self.run_decode_graph(seqs), temperatures)
             reset_context()
             return token_ids
         input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
         temperatures = self.prepare_sample(seqs)
-        logits = self.run_model(input_ids, positions, is_prefill)
-        token_ids = self.sampler(logits, temperatures, self._all_greedy).tolist()   # the step's one device sync
+        token_ids = self.sample(self.run_hidden(input_ids, positions, is_prefill), temperatures)
         reset_context()
         return token_ids
 

@@ -34,3 +34,12 @@ class ParallelLMHead(VocabParallelEmbedding):
             last = (ctx.cu_seqlens_q[1:] - 1).long()
             x = x[last].contiguous()
         return ops.bf16_linear(x, self.weight.data)
+
+    def forward_greedy(self, x: torch.Tensor):
+        """``argmax(self(x), -1)``: the greedy branch of the sampler (sampler.py:13-14,21) applied to this
+        layer's logits, in one call that never stores them."""
+        ctx = get_context()
+        if ctx.is_prefill:
+            last = (ctx.cu_seqlens_q[1:] - 1).long()
+            x = x[last].contiguous()
+        return ops.bf16_linear_argmax(x, self.weight.data)

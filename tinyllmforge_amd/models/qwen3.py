@@ -160,6 +160,10 @@ class Qwen3ForCausalLM(nn.Module):
     def compute_logits(self, hidden_states: torch.Tensor) -> torch.Tensor:
         return self.lm_head(hidden_states)
 
+    def compute_greedy_ids(self, hidden_states: torch.Tensor) -> torch.Tensor:
+        """Token ids of an all-greedy batch: LM head and argmax in one call, no logits in memory."""
+        return self.lm_head.forward_greedy(hidden_states)
+
     def quantize_linears_(self):
         """Weight-only int8 for the four projections of every layer (embedding and LM head stay bf16)."""
         for layer in self.model.layers:

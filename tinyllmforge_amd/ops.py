@@ -249,6 +249,20 @@ def bf16_linear(x, w):
     return y.view(*x.shape[:-1], N)
 
 
+def bf16_linear_argmax(x, w):
+    """``argmax(bf16_linear(x, w), -1)`` (first index among ties) without the logits: int64 ``[M]``."""
+    lib = _lib.load()
+    _need(x, BF16, "x"); _need(w, BF16, "w")
+    assert x.stride(-1) == 1 and w.is_contiguous() and x.dim() == 2
+    M, K = x.shape
+    N = w.shape[0]
+    out = torch.empty(M, dtype=torch.int64, device=x.device)
+    ws = _workspace(lib.tlf_gemm_argmax_workspace_bytes(M, N, K), x.device, "gemm")
+    check(lib.tlf_bf16_gemm_argmax(x.data_ptr(), x.stride(0), w.data_ptr(), out.data_ptr(), M, N, K,
+                                   ws.data_ptr(), ws.numel(), _stream()), "tlf_bf16_gemm_argmax")
+    return out
+
+
 def linear_add_rms_norm(x, w, scale, residual, norm_weight, eps):
     """``add_rms_norm(linear(x), residual)`` behind one call: ``w`` int8 with ``scale`` (weight-only int8)
     or bf16 with ``scale=None``.  Returns ``(normed, new_residual)``, the bits of the two separate calls."""
