@@ -326,6 +326,18 @@ def bench_e2e(args, quantization):
         stats["decode_byte_floor"] = decode_byte_floor(llm.config.hf_config, llm.last_stats, quantization, kv_itemsize=2)
     res = dict(tok_s=total / wall, wall_s=wall, total_output_tokens=total, init_s=round(init_s, 1), stats=stats,
                kv_blocks=llm.config.num_kvcache_blocks)
+    if quantization is not None and args.steps == 0:
+        # the reference's script samples at temperature 0.6 (bench.py:49): same workload through the
+        # logits + sampling-kernel path instead of the fused LM head + argmax
+        hot = [SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=m) for m in max_tokens]
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        llm.generate(prompts, hot)
+        torch.cuda.synchronize()
+        w = time.perf_counter() - t0
+        res["temperature_0.6"] = dict(tok_s=round(total / w, 1), wall_s=round(w, 3),
+                                      decode_ms_per_step=round(1e3 * llm.last_stats["decode_time"] /
+                                                               max(1, llm.last_stats["decode_steps"]), 3))
     cpu = None
     if quantization is None and not args.no_cpu_baseline:
         cpu = cpu_baseline_e2e(llm, prompts)

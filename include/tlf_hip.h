@@ -167,6 +167,23 @@ int tlf_argmax(const void *logits, int64_t row_stride, int64_t *out,
                int32_t rows, int32_t vocab, void *workspace, size_t workspace_bytes,
                void *stream);
 
+/* Sampler.forward with temperatures   replaces layers/sampler.py:13-21
+ *
+ *   T[b] == 0:  out[b] = first index of max(logits[b, :])
+ *   T[b]  > 0:  out[b] = argmax_i softmax(logits[b, :] / T[b])_i / (e_i + 1e-10),  e_i ~ Exp(1)
+ *               computed as argmax_i logits[b, i] / T[b] - log(e_i + 1e-10)  (same index: the row's
+ *               normaliser is common and log is monotone), one pass over the row.
+ *
+ * The reference takes e from torch's device generator, whose stream no kernel can reproduce; here
+ * e_i = -log(u_i) with u from Philox4x32-10: key = seed, counter = (i / 4, b, offset) gives the
+ * uniforms of elements 4 (i / 4) .. + 3, u = (x >> 8) * 2^-24 + 2^-25.  Same distribution, its
+ * own stream; the caller advances offset once per call.
+ * logits bf16 [rows, vocab] (row stride in elements), temperatures fp32 [rows] >= 0, out int64
+ * [rows].  workspace: tlf_argmax_workspace_bytes(rows, vocab). */
+int tlf_sample(const void *logits, int64_t row_stride, const float *temperatures, int64_t *out,
+               int32_t rows, int32_t vocab, uint64_t seed, uint64_t offset,
+               void *workspace, size_t workspace_bytes, void *stream);
+
 /* ---------------------------------------------------------------------------
  * a10  weight-only int8 linear (build-defined; the reference has bf16 F.linear
  * only: layers/linear.py:48-49, 82-83, 180-181; same [N, K] weight layout)

@@ -129,6 +129,50 @@ def greedy_sample(logits):
     return logits.to(torch.float32).argmax(dim=-1)
 
 
+def philox4x32_10(counter, key):
+    """Philox4x32-10 (Salmon, Moraes, Dror, Shaw: "Parallel random numbers: as easy as 1, 2, 3", SC'11;
+    the Random123 library).  ``counter`` uint32 ``[..., 4]``, ``key`` two uint32 -> uint32 ``[..., 4]``."""
+    import numpy as np
+    c = [np.asarray(counter[..., i], dtype=np.uint64) for i in range(4)]
+    k0, k1 = int(key[0]), int(key[1])
+    mask = np.uint64(0xFFFFFFFF)
+    for _ in range(10):
+        p0 = np.uint64(0xD2511F53) * c[0]
+        p1 = np.uint64(0xCD9E8D57) * c[2]
+        c = [(p1 >> np.uint64(32)) ^ c[1] ^ np.uint64(k0), p1 & mask,
+             (p0 >> np.uint64(32)) ^ c[3] ^ np.uint64(k1), p0 & mask]
+        k0, k1 = (k0 + 0x9E3779B9) & 0xFFFFFFFF, (k1 + 0xBB67AE85) & 0xFFFFFFFF
+    return np.stack(c, -1).astype(np.uint32)
+
+
+def sample_scores(logits, temperatures, seed, offset):
+    """Build-defined noise for tinyvllm/layers/sampler.py:15-20.  The reference's
+    ``argmax(softmax(l / T) / (e + 1e-10))`` with ``e ~ Exp(1)`` equals ``argmax(l / T - log(e + 1e-10))``
+    (common normaliser, monotone log); ``e = -log(u)``, ``u = (x >> 8) 2^-24 + 2^-25`` with ``x`` the
+    Philox word of (key = seed, counter = (i // 4, row, offset), word i % 4).  Rows with T == 0 keep their
+    logits.  Returns the fp32 scores ``[rows, vocab]``; the sample is their first argmax."""
+    import numpy as np
+    l = logits.to(torch.float32).numpy()
+    t = np.asarray(temperatures, dtype=np.float32)
+    rows, vocab = l.shape
+    nq = (vocab + 3) // 4
+    ctr = np.zeros((rows, nq, 4), dtype=np.uint32)
+    ctr[..., 0] = np.arange(nq, dtype=np.uint32)[None, :]
+    ctr[..., 1] = np.arange(rows, dtype=np.uint32)[:, None]
+    ctr[..., 2] = offset & 0xFFFFFFFF
+    ctr[..., 3] = (offset >> 32) & 0xFFFFFFFF
+    x = philox4x32_10(ctr, (seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF)).reshape(rows, nq * 4)[:, :vocab]
+    u = (x >> np.uint32(8)).astype(np.float32) * np.float32(2.0 ** -24) + np.float32(2.0 ** -25)
+    e = -np.log(u, dtype=np.float32)
+    safe_t = np.where(t == 0, np.float32(1), t)[:, None]
+    noisy = l / safe_t - np.log(e + np.float32(1e-10), dtype=np.float32)
+    return torch.from_numpy(np.where((t == 0)[:, None], l, noisy).astype(np.float32))
+
+
+def sample(logits, temperatures, seed, offset):
+    return sample_scores(logits, temperatures, seed, offset).argmax(dim=-1)
+
+
 # --------------------------------------------------------------------------- a10
 def linear(x, weight, bias=None):
     """tinyvllm/layers/linear.py:48-49, 82-83, 180-181: ``bf16(sum_k x[m,k] W[n,k])``."""

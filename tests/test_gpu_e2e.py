@@ -165,6 +165,22 @@ def test_fused_lm_head_argmax_gives_the_tokens_of_logits_then_sampler(llm_c1):
     assert a == b
 
 
+def test_mixed_temperatures_keep_the_greedy_rows_and_sample_the_others(llm_c1):
+    """A batch with temperatures [0, 0.8, 0, 1.2] goes through logits and the sampling kernel: its greedy rows
+    produce the tokens of the all-greedy run (the fused LM head + argmax path), the sampled rows other tokens
+    from the vocabulary."""
+    from tinyllmforge_amd import SamplingParams
+    prompts = [p[:64] for p in c1_prompts()]
+    greedy = SamplingParams(temperature=0.0, max_tokens=10, ignore_eos=True)
+    a = [o["token_ids"] for o in llm_c1.generate(prompts, greedy)]
+    sps = [SamplingParams(temperature=t, max_tokens=10, ignore_eos=True) for t in (0.0, 0.8, 0.0, 1.2)]
+    b = [o["token_ids"] for o in llm_c1.generate(prompts, sps)]
+    assert b[0] == a[0] and b[2] == a[2]
+    assert b[1] != a[1] and b[3] != a[3]
+    vocab = llm_c1.model_runner.config.hf_config.vocab_size
+    assert all(0 <= tok < vocab for row in b for tok in row)
+
+
 def test_unfused_layer_path_gives_identical_tokens(llm_c1):
     from tinyllmforge_amd import SamplingParams
     sp = SamplingParams(temperature=0.0, max_tokens=6, ignore_eos=True)

@@ -216,6 +216,41 @@ def test_argmax_all_negative_and_zero_signs(ops):
     assert ops.argmax(l.to(DEV)).tolist() == O.greedy_sample(l).tolist() == [40, 63]
 
 
+# ----------------------------------------------------------------------------- sampler with temperatures
+@pytest.mark.parametrize("rows,vocab", [(7, 1003), (64, 151936), (3, 8)])
+def test_sample_matches_the_oracle_on_the_same_philox_stream(ops, rows, vocab):
+    """Same seed and offset, same Philox words: the kernel's choice must be the oracle's, except where
+    the oracle's two best scores are closer than the last ulps of logf (then either of them)."""
+    pad = (-vocab) % 8
+    buf = (torch.randn(rows, vocab + pad, generator=g(rows + vocab)) * 2).to(BF)
+    logits = buf[:, :vocab]
+    t = torch.tensor([0.0, 0.6, 1.0, 2.5] * rows)[:rows].contiguous()
+    for seed, offset in ((0, 1), (12345678901234, 2 ** 33 + 5)):
+        got = ops.sample(buf.to(DEV)[:, :vocab], t.to(DEV), seed, offset).cpu()
+        sc = O.sample_scores(logits, t, seed, offset)
+        ref = sc.argmax(-1)
+        assert torch.equal(got[t == 0], O.greedy_sample(logits)[t == 0])
+        same = got == ref
+        chosen = sc.gather(1, got[:, None])[:, 0]
+        top = sc.max(-1).values
+        assert ((top - chosen) <= 8 * torch.finfo(torch.float32).eps * top.abs().clamp_min(1.0)).all()
+        assert same.float().mean().item() >= 0.95
+    assert not torch.equal(ops.sample(buf.to(DEV)[:, :vocab], t.to(DEV), 0, 1).cpu()[t > 0],
+                           ops.sample(buf.to(DEV)[:, :vocab], t.to(DEV), 0, 2).cpu()[t > 0]) or rows < 4
+
+
+def test_sample_follows_softmax(ops):
+    """32768 rows with the same 16 logits at T = 0.8: chi-square of the kernel's draws against
+    softmax(l / T), 15 degrees of freedom, bound 45 (p ~ 1e-4)."""
+    row = torch.tensor([2.0, 1.0, 0.5, 0.0, -0.5, -1.0, 1.5, -3.0, 0.25, 0.75, -2.0, 1.25, -0.25, 0.1, -1.5, 1.75])
+    logits = row.to(BF)[None, :].repeat(32768, 1).contiguous()
+    t = torch.full((32768,), 0.8)
+    draws = ops.sample(logits.to(DEV), t.to(DEV), 3, 9).cpu()
+    want = torch.softmax(logits[0].double() / 0.8, -1) * 32768
+    got = torch.bincount(draws, minlength=16).double()
+    assert (((got - want) ** 2) / want).sum().item() < 45
+
+
 # ----------------------------------------------------------------------------- K9
 def test_embedding_bit_exact(ops):
     w = torch.randn(1000, 1024, generator=g(0)).to(BF)

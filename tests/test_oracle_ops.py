@@ -153,6 +153,50 @@ def test_greedy_sample_ties_take_first_index():
 
 
 # ---------------------------------------------------------------- linear / w8a16
+def test_philox4x32_10_known_answers():
+    """The three known-answer vectors of the Random123 distribution (kat_vectors, philox4x32 10)."""
+    kats = [((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
+            ((0xffffffff,) * 4, (0xffffffff,) * 2, (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
+            ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0),
+             (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1))]
+    for ctr, key, want in kats:
+        got = O.philox4x32_10(np.array(ctr, dtype=np.uint32), key)
+        assert tuple(int(v) for v in got) == want
+    both = O.philox4x32_10(np.array([kats[0][0], kats[2][0]], dtype=np.uint32)[:, None, :].repeat(3, 1), (0, 0))
+    assert both.shape == (2, 3, 4) and tuple(int(v) for v in both[0, 2]) == kats[0][2]      # batched counters
+
+
+def test_sample_is_the_reference_formula_on_the_same_noise_and_follows_softmax():
+    """(1) T == 0 rows keep their logits (greedy, first index).  (2) On the noise the oracle draws, its choice
+    maximises the reference's own expression softmax(l/T) / (e + 1e-10) (sampler.py:15-20) evaluated in fp64.
+    (3) 40000 independent draws from one row follow softmax(l/T): chi-square over 8 tokens, 7 degrees of
+    freedom, bound 30 (p ~ 1e-4).  (4) other offsets and seeds give other draws."""
+    l = (torch.randn(64, 1003, generator=g(5)) * 2).to(BF)
+    t = torch.tensor([0.0, 0.5, 1.0, 2.0] * 16)
+    sc = O.sample_scores(l, t, seed=7, offset=3)
+    assert torch.equal(sc[0::4], l[0::4].float())
+    ids = O.sample(l, t, 7, 3)
+    assert torch.equal(ids[0::4], O.greedy_sample(l[0::4]))
+    # recover e from the scores' definition independently: same Philox words, fp64 arithmetic
+    rows, vocab = l.shape
+    ctr = np.zeros((rows, (vocab + 3) // 4, 4), dtype=np.uint32)
+    ctr[..., 0] = np.arange(ctr.shape[1])[None, :]; ctr[..., 1] = np.arange(rows)[:, None]; ctr[..., 2] = 3
+    x = O.philox4x32_10(ctr, (7, 0)).reshape(rows, -1)[:, :vocab]
+    e = -np.log((x >> 8).astype(np.float64) * 2.0 ** -24 + 2.0 ** -25)
+    for r in range(rows):
+        if t[r] == 0:
+            continue
+        p = torch.softmax(l[r].double() / float(t[r]), -1).numpy() / (e[r] + 1e-10)
+        assert p[ids[r]] >= p.max() * (1 - 1e-5), r
+    logits = torch.tensor([[2.0, 1.0, 0.5, 0.0, -0.5, -1.0, 1.5, -3.0]]).to(BF).repeat(40000, 1)
+    draws = O.sample(logits, torch.full((40000,), 0.7), seed=1, offset=0)
+    want = torch.softmax(logits[0].double() / 0.7, -1) * 40000
+    got = torch.bincount(draws, minlength=8).double()
+    assert (((got - want) ** 2) / want).sum().item() < 30
+    assert not torch.equal(draws, O.sample(logits, torch.full((40000,), 0.7), seed=1, offset=1))
+    assert not torch.equal(draws, O.sample(logits, torch.full((40000,), 0.7), seed=2, offset=0))
+
+
 def test_linear_matches_fp64():
     x = torch.randn(5, 64, generator=g(13)).to(BF)
     w = (torch.randn(24, 64, generator=g(14)) * 0.1).to(BF)

@@ -8,7 +8,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_float, c_int32, c_int64, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int32, c_int64, c_size_t, c_uint64, c_void_p
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtlf_hip.so")
@@ -34,6 +34,7 @@ SIGNATURES = {
     "tlf_silu_and_mul": (c_int32, [_P, _P, _I32, _I32, _P]),
     "tlf_argmax_workspace_bytes": (_SZ, [_I32, _I32]),
     "tlf_argmax": (c_int32, [_P, _I64, _P, _I32, _I32, _P, _SZ, _P]),
+    "tlf_sample": (c_int32, [_P, _I64, _P, _P, _I32, _I32, c_uint64, c_uint64, _P, _SZ, _P]),
     "tlf_w8a16_gemm_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
     "tlf_w8a16_gemm": (c_int32, [_P, _I64, _P, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),
     "tlf_bf16_gemm": (c_int32, [_P, _I64, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),

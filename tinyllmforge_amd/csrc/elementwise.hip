@@ -300,6 +300,98 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(
   if (threadIdx.x == 0) out[row] = static_cast<int64_t>(0xffffffffu - static_cast<unsigned int>(best));
 }
 
+// --------------------------------------------------------------------------
+// Sampler with temperatures (reference: tinyvllm/layers/sampler.py:13-20).
+//   T == 0:  first index of the largest logit
+//   T  > 0:  argmax_i softmax(l / T)_i / (e_i + 1e-10),  e_i ~ Exp(1)
+// The softmax normaliser is common to a row and log is monotone, so the sampled index is
+//   argmax_i  l_i / T - log(e_i + 1e-10),   e_i = -log(u_i)
+// in one pass over the row, with no exp and no row sum.  The reference draws e from torch's
+// device generator; here u comes from Philox4x32-10 (Salmon et al., SC'11) keyed by the caller's
+// seed: counter = (i / 4, row, offset_lo, offset_hi) yields the uniforms of elements 4*(i/4)..+3,
+// u = (x >> 8) * 2^-24 + 2^-25 in (0, 1).  Same law, a stream of its own.
+__device__ __forceinline__ void philox4x32_10(unsigned int (&c)[4], unsigned int k0, unsigned int k1) {
+#pragma unroll
+  for (int round = 0; round < 10; ++round) {
+    const unsigned long long p0 = 0xD2511F53ull * c[0];
+    const unsigned long long p1 = 0xCD9E8D57ull * c[2];
+    const unsigned int n0 = static_cast<unsigned int>(p1 >> 32) ^ c[1] ^ k0;
+    const unsigned int n2 = static_cast<unsigned int>(p0 >> 32) ^ c[3] ^ k1;
+    c[1] = static_cast<unsigned int>(p1);
+    c[3] = static_cast<unsigned int>(p0);
+    c[0] = n0;
+    c[2] = n2;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+}
+
+// key of an fp32 score: order-preserving image of the value << 32 | ~index (cf. argmax_key)
+__device__ __forceinline__ unsigned long long score_key(float v, unsigned int idx) {
+  v += 0.0f;  // -0 -> +0
+  const unsigned int b = __float_as_uint(v);
+  const unsigned int ord = (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+  return (static_cast<unsigned long long>(ord) << 32) | (0xffffffffu - idx);
+}
+
+__device__ __forceinline__ float sample_score(float logit, float temp, unsigned int x) {
+  if (temp == 0.f) return logit;
+  const float u = static_cast<float>(x >> 8) * 0x1p-24f + 0x1p-25f;
+  const float e = -logf(u);
+  return __fsub_rn(__fdiv_rn(logit, temp), logf(__fadd_rn(e, 1e-10f)));
+}
+
+__global__ __launch_bounds__(256) void sample_partial_kernel(
+    const unsigned short *__restrict__ logits, int64_t row_stride, int32_t vocab,
+    const float *__restrict__ temperatures, unsigned int seed_lo, unsigned int seed_hi,
+    unsigned int off_lo, unsigned int off_hi, unsigned long long *__restrict__ partial,
+    int32_t nchunks) {
+  const int row = blockIdx.y;
+  const int chunk = blockIdx.x;
+  const unsigned short *lr = logits + row * row_stride;
+  const float temp = temperatures[row];
+  const int nvec = vocab / 8;
+  const int vec_per_chunk = (nvec + nchunks - 1) / nchunks;
+  const int v0 = chunk * vec_per_chunk;
+  const int v1 = min(v0 + vec_per_chunk, nvec);
+  unsigned long long best = 0;
+  for (int v = v0 + threadIdx.x; v < v1; v += blockDim.x) {
+    const uint4 p = *reinterpret_cast<const uint4 *>(lr + static_cast<int64_t>(v) * 8);
+    float l[8];
+    unpack8(p, l);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      unsigned int c[4] = {static_cast<unsigned int>(v * 2 + h), static_cast<unsigned int>(row), off_lo, off_hi};
+      if (temp != 0.f) philox4x32_10(c, seed_lo, seed_hi);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const unsigned long long key = score_key(sample_score(l[h * 4 + i], temp, c[i]),
+                                                 static_cast<unsigned int>(v * 8 + h * 4 + i));
+        best = key > best ? key : best;
+      }
+    }
+  }
+  if (chunk == 0) {  // scalar tail when vocab is not a multiple of 8
+    const int t = nvec * 8 + threadIdx.x;
+    if (t < vocab) {
+      unsigned int c[4] = {static_cast<unsigned int>(t / 4), static_cast<unsigned int>(row), off_lo, off_hi};
+      if (temp != 0.f) philox4x32_10(c, seed_lo, seed_hi);
+      const unsigned int x = (t & 3) == 0 ? c[0] : (t & 3) == 1 ? c[1] : (t & 3) == 2 ? c[2] : c[3];
+      const unsigned long long key =
+          score_key(sample_score(bf16_bits_to_float(lr[t]), temp, x), static_cast<unsigned int>(t));
+      best = key > best ? key : best;
+    }
+  }
+  __shared__ unsigned long long part[4];
+  best = wave_max_u64(best);
+  if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = best;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < 4; ++w) best = part[w] > best ? part[w] : best;
+    partial[static_cast<int64_t>(row) * nchunks + chunk] = best;
+  }
+}
+
 // Last stage of the greedy sample on its own: rows x nparts keys (argmax_key) -> token ids.
 int launch_argmax_final(const unsigned long long *keys, int32_t nparts, int64_t *out, int32_t rows,
                         hipStream_t stream) {
@@ -456,6 +548,28 @@ extern "C" int tlf_argmax(const void *logits, int64_t row_stride, int64_t *out, 
   hipLaunchKernelGGL(argmax_partial_kernel, dim3(nchunks, rows), dim3(256), 0,
                      static_cast<hipStream_t>(stream),
                      static_cast<const unsigned short *>(logits), row_stride, vocab, part, nchunks);
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(64), 0,
+                     static_cast<hipStream_t>(stream), part, nchunks, out);
+  return launch_status();
+}
+
+extern "C" int tlf_sample(const void *logits, int64_t row_stride, const float *temperatures,
+                          int64_t *out, int32_t rows, int32_t vocab, uint64_t seed, uint64_t offset,
+                          void *workspace, size_t workspace_bytes, void *stream) {
+  if (rows == 0) return TLF_OK;
+  if (!logits || !out || !temperatures) return TLF_E_NULL;
+  if (rows < 0 || vocab <= 0 || row_stride < vocab) return TLF_E_SHAPE;
+  if (!aligned16(logits) || row_stride % 8) return TLF_E_ALIGN;
+  if (!workspace || workspace_bytes < tlf_argmax_workspace_bytes(rows, vocab) ||
+      (reinterpret_cast<uintptr_t>(workspace) & 7u))
+    return TLF_E_WORKSPACE;
+  const int nchunks = argmax_chunks(rows, vocab);
+  auto part = static_cast<unsigned long long *>(workspace);
+  hipLaunchKernelGGL(sample_partial_kernel, dim3(nchunks, rows), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const unsigned short *>(logits),
+                     row_stride, vocab, temperatures, static_cast<unsigned int>(seed),
+                     static_cast<unsigned int>(seed >> 32), static_cast<unsigned int>(offset),
+                     static_cast<unsigned int>(offset >> 32), part, nchunks);
   hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(64), 0,
                      static_cast<hipStream_t>(stream), part, nchunks, out);
   return launch_status();

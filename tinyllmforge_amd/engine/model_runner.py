@@ -53,7 +53,7 @@ class ModelRunner:
         finally:
             torch.set_default_dtype(default_dtype)
         self.model.eval()
-        self.sampler = Sampler()
+        self.sampler = Sampler(seed=config.seed)
         self.fused_greedy = True      # all-greedy batches: LM head and argmax in one call
         self.graphs = {}
         self.graph_bs = []

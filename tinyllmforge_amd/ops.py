@@ -179,6 +179,23 @@ def argmax(logits):
     return out
 
 
+def sample(logits, temperatures, seed: int, offset: int):
+    """Sampler with temperatures: greedy where ``temperatures == 0``, else one draw from
+    ``softmax(logits / T)`` by the exponential-race formula of the reference, noise from Philox4x32-10
+    at (``seed``, ``offset``).  int64 ``[rows]``."""
+    lib = _lib.load()
+    _need(logits, BF16, "logits"); _need(temperatures, torch.float32, "temperatures")
+    assert logits.dim() == 2 and logits.stride(1) == 1 and temperatures.is_contiguous()
+    rows, vocab = logits.shape
+    assert temperatures.numel() == rows
+    out = torch.empty(rows, dtype=torch.int64, device=logits.device)
+    ws = _workspace(lib.tlf_argmax_workspace_bytes(rows, vocab), logits.device, "argmax")
+    check(lib.tlf_sample(logits.data_ptr(), logits.stride(0), temperatures.data_ptr(), out.data_ptr(), rows,
+                         vocab, seed & (2 ** 64 - 1), offset & (2 ** 64 - 1), ws.data_ptr(), ws.numel(),
+                         _stream()), "tlf_sample")
+    return out
+
+
 # ------------------------------------------------------------------ K9
 def embedding(ids, weight):
     lib = _lib.load()
