@@ -248,3 +248,58 @@ def test_gate_up_interleave_index_is_the_stated_permutation():
         for j in range(0, n, 16):
             assert idx[j:j + 8].tolist() == list(range(j // 2, j // 2 + 8))
             assert idx[j + 8:j + 16].tolist() == list(range(half + j // 2, half + j // 2 + 8))
+
+
+def test_safetensors_loader_and_offline_int8_checkpoint(tmp_path):
+    """Weights on disk (loader.py:11-30): an HF-style checkpoint with q/k/v and gate/up stored apart loads
+    into the packed parameters; the offline quantiser's int8 checkpoint loads to exactly the int8 weights,
+    scales and gate/up row order that quantising the loaded bf16 model in memory gives."""
+    import torch
+    from safetensors.torch import save_file
+    from tinyllmforge_amd.models.qwen3 import Qwen3ForCausalLM
+    from tinyllmforge_amd.utils.loader import load_model, quantize_checkpoint, random_init_
+    cfg = ModelConfig.from_any(dict(hidden_size=128, num_hidden_layers=2, num_attention_heads=2, num_key_value_heads=1,
+                                     head_dim=64, intermediate_size=96, vocab_size=200, max_position_embeddings=64,
+                                     tie_word_embeddings=False))
+    torch.set_default_dtype(torch.bfloat16)
+    try:
+        src = random_init_(Qwen3ForCausalLM(cfg), seed=3)
+        a, b = Qwen3ForCausalLM(cfg), Qwen3ForCausalLM(cfg)
+    finally:
+        torch.set_default_dtype(torch.float32)
+    # unpack the way a HF checkpoint stores it, split over two files
+    hf = {}
+    for name, p in src.named_parameters():
+        t = p.data
+        if "qkv_proj" in name:
+            attn = src.get_submodule(name.rsplit(".", 2)[0])
+            q, k, v = t.split([attn.q_size, attn.kv_size, attn.kv_size], 0)
+            for key, part in (("q_proj", q), ("k_proj", k), ("v_proj", v)):
+                hf[name.replace("qkv_proj", key)] = part.contiguous()
+        elif "gate_up_proj" in name:
+            gate, up = t.chunk(2, 0)
+            hf[name.replace("gate_up_proj", "gate_proj")] = gate.contiguous()
+            hf[name.replace("gate_up_proj", "up_proj")] = up.contiguous()
+        else:
+            hf[name] = t.contiguous()
+    names = sorted(hf)
+    d16, d8 = tmp_path / "bf16", tmp_path / "int8"
+    d16.mkdir()
+    save_file({n: hf[n] for n in names[::2]}, str(d16 / "model-00001-of-00002.safetensors"))
+    save_file({n: hf[n] for n in names[1::2]}, str(d16 / "model-00002-of-00002.safetensors"))
+    load_model(a, str(d16))
+    for (n1, p1), (n2, p2) in zip(src.named_parameters(), a.named_parameters()):
+        assert n1 == n2 and torch.equal(p1.data, p2.data), n1
+    quantize_checkpoint(str(d16), str(d8))
+    load_model(b, str(d8))
+    a.quantize_linears_()
+    b.quantize_linears_()                       # nothing left to do for a checkpoint that is int8 already
+    for la, lb in zip(a.model.layers, b.model.layers):
+        for get in (lambda l: l.self_attn.qkv_proj, lambda l: l.self_attn.o_proj,
+                    lambda l: l.mlp.gate_up_proj, lambda l: l.mlp.down_proj):
+            ma, mb = get(la), get(lb)
+            assert mb.qweight.dtype == torch.int8 and mb.weight.numel() == 0
+            assert torch.equal(ma.qweight, mb.qweight) and torch.equal(ma.qscale, mb.qscale)
+        assert la.mlp.gate_up_proj.interleaved and lb.mlp.gate_up_proj.interleaved
+    assert torch.equal(a.model.embed_tokens.weight, b.model.embed_tokens.weight)
+    assert torch.equal(a.lm_head.weight, b.lm_head.weight) and torch.equal(a.model.norm.weight, b.model.norm.weight)

@@ -41,7 +41,10 @@ class LinearBase(nn.Module):
             self.register_parameter("bias", None)
 
     def quantize_(self):
-        """Replace the bf16 weight by int8 + scale (frees the bf16 copy)."""
+        """Replace the bf16 weight by int8 + scale (frees the bf16 copy).  Nothing to do for a layer
+        whose int8 weight came from a quantised checkpoint."""
+        if self.qweight is not None:
+            return self
         self.qweight, self.qscale = quantize_per_channel(self.weight.data)
         self.weight.data = torch.empty(0, dtype=self.weight.dtype, device=self.weight.device)
         return self
@@ -49,6 +52,30 @@ class LinearBase(nn.Module):
     def load_quantized(self, qweight: torch.Tensor, qscale: torch.Tensor):
         self.qweight, self.qscale = qweight.contiguous(), qscale.contiguous()
         self.weight.data = torch.empty(0, dtype=self.weight.dtype, device=qweight.device)
+
+    def shard_rows(self, shard_id=None):
+        """(first output row, row count) of a checkpoint tensor inside this layer's weight."""
+        return 0, self.weight.shape[0] if self.weight.numel() else self.qweight.shape[0]
+
+    def load_quantized_shard(self, kind: str, tensor: torch.Tensor, shard_id=None):
+        """One ``.qweight`` (int8 ``[rows, in]``) or ``.qscale`` (fp32 ``[rows]``) tensor of a quantised
+        checkpoint into rows ``shard_rows(shard_id)``.  Per-output-channel scales make the rows of a packed
+        projection independent, so q/k/v (gate/up) are quantised one by one offline and packed here."""
+        if self.qweight is None:
+            out_f, in_f = self.weight.shape
+            dev = self.weight.device
+            self.qweight = torch.zeros(out_f, in_f, dtype=torch.int8, device=dev)
+            self.qscale = torch.ones(out_f, dtype=torch.float32, device=dev)
+            self.weight.data = torch.empty(0, dtype=self.weight.dtype, device=dev)
+            self.pending_quantized = True
+        first, rows = self.shard_rows(shard_id)
+        dst = self.qweight if kind == "qweight" else self.qscale
+        assert tensor.shape[0] == rows and tensor.dtype == dst.dtype, (kind, tensor.shape, tensor.dtype)
+        dst[first:first + rows].copy_(tensor)
+
+    def finish_quantized_load(self):
+        """Called once after every shard is in."""
+        self.pending_quantized = False
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self.qweight is not None:
@@ -91,14 +118,26 @@ class MergedColumnParallelLinear(ColumnParallelLinear):
     def quantize_(self):
         """int8 + scale; a gate/up pair is also re-ordered for the fused projection + SiLU-and-mul
         kernel (``ops.gate_up_interleave_index``), which ``forward_silu_mul`` then uses."""
-        super().quantize_()
-        if len(self.output_sizes) == 2 and self.output_sizes[0] == self.output_sizes[1] \
+        if self.qweight is None:
+            super().quantize_()
+            self.interleave_()
+        return self
+
+    def interleave_(self):
+        if not getattr(self, "interleaved", False) and len(self.output_sizes) == 2 \
+                and self.output_sizes[0] == self.output_sizes[1] \
                 and sum(self.output_sizes) % 16 == 0 and self.bias is None:
             idx = ops.gate_up_interleave_index(sum(self.output_sizes), self.qweight.device)
             self.qweight = self.qweight[idx].contiguous()
             self.qscale = self.qscale[idx].contiguous()
             self.interleaved = True
-        return self
+
+    def shard_rows(self, shard_id=None):
+        return sum(self.output_sizes[:shard_id]) // self.tp_size, self.output_sizes[shard_id] // self.tp_size
+
+    def finish_quantized_load(self):
+        super().finish_quantized_load()
+        self.interleave_()
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if getattr(self, "interleaved", False):
@@ -130,10 +169,13 @@ class QKVParallelLinear(ColumnParallelLinear):
         self.num_kv_heads = self.total_num_kv_heads
         super().__init__(hidden_size, (self.num_heads + 2 * self.num_kv_heads) * head_size, bias)
 
-    def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor, loaded_shard_id: str):
-        assert loaded_shard_id in ("q", "k", "v")
+    def shard_rows(self, shard_id=None):
+        assert shard_id in ("q", "k", "v")
         q_size, kv_size = self.num_heads * self.head_size, self.num_kv_heads * self.head_size
-        offset, size = {"q": (0, q_size), "k": (q_size, kv_size), "v": (q_size + kv_size, kv_size)}[loaded_shard_id]
+        return {"q": (0, q_size), "k": (q_size, kv_size), "v": (q_size + kv_size, kv_size)}[shard_id]
+
+    def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor, loaded_shard_id: str):
+        offset, size = self.shard_rows(loaded_shard_id)
         dst = param.data.narrow(self.tp_dim, offset, size)
         dst.copy_(loaded_weight.chunk(self.tp_size, self.tp_dim)[self.tp_rank])
 

@@ -1,5 +1,6 @@
-"""Weights into a model: safetensors files (reference: tinyvllm/utils/loader.py:11-30) or a
-seeded random initialisation for the benchmark / parity configurations."""
+"""Weights into a model: safetensors files (reference: tinyvllm/utils/loader.py:11-30), bf16 or
+quantised offline by ``quantize_checkpoint``, or a seeded random initialisation for the benchmark /
+parity configurations."""
 from __future__ import annotations
 
 import os
@@ -22,9 +23,19 @@ def load_model(model: nn.Module, path: str):
         with safe_open(file, "pt", "cpu") as f:
             for name in f.keys():
                 load_tensor(model, packed, name, f.get_tensor(name))
+    finish_load(model)
 
 
 def load_tensor(model: nn.Module, packed: dict, name: str, tensor: torch.Tensor):
+    kind = name.rsplit(".", 1)[-1]
+    if kind in ("qweight", "qscale"):          # a checkpoint written by quantize_checkpoint
+        module_name, shard_id = name.rsplit(".", 1)[0], None
+        for key, (target, sid) in packed.items():
+            if key in module_name:
+                module_name, shard_id = module_name.replace(key, target), sid
+                break
+        model.get_submodule(module_name).load_quantized_shard(kind, tensor, shard_id)
+        return
     for key, (target, shard_id) in packed.items():
         if key in name:
             param = model.get_parameter(name.replace(key, target))
@@ -34,11 +45,49 @@ def load_tensor(model: nn.Module, packed: dict, name: str, tensor: torch.Tensor)
     getattr(param, "weight_loader", default_weight_loader)(param, tensor)
 
 
+def finish_load(model: nn.Module):
+    for m in model.modules():
+        if getattr(m, "pending_quantized", False):
+            m.finish_quantized_load()
+
+
+QUANTIZED_SUFFIXES = ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj")
+
+
+def quantize_checkpoint(src: str, dst: str):
+    """Offline weight-only int8: every ``*_proj.weight`` of ``src/*.safetensors`` becomes ``*.qweight`` (int8,
+    same ``[out, in]`` layout) plus ``*.qscale`` (fp32 ``[out]``, ``max|row| / 127``) in ``dst``; every other
+    tensor is copied.  Rows are independent, so the unpacked q/k/v and gate/up tensors quantise to exactly
+    the rows that quantising the packed weight gives.  Streams one file at a time."""
+    from safetensors import safe_open
+    from safetensors.torch import save_file
+    from ..layers.linear import quantize_per_channel
+    os.makedirs(dst, exist_ok=True)
+    for file in sorted(glob(os.path.join(src, "*.safetensors"))):
+        out = {}
+        with safe_open(file, "pt", "cpu") as f:
+            for name in f.keys():
+                t = f.get_tensor(name)
+                stem = name[:-len(".weight")] if name.endswith(".weight") else None
+                if stem is not None and stem.rsplit(".", 1)[-1] in QUANTIZED_SUFFIXES and t.dim() == 2:
+                    wq, scale = quantize_per_channel(t)
+                    out[stem + ".qweight"], out[stem + ".qscale"] = wq, scale
+                else:
+                    out[name] = t.contiguous()
+        save_file(out, os.path.join(dst, os.path.basename(file)))
+    for extra in ("config.json",):
+        p = os.path.join(src, extra)
+        if os.path.exists(p):
+            import shutil
+            shutil.copy(p, os.path.join(dst, extra))
+
+
 def load_state_dict(model: nn.Module, state: dict):
     """Same routing as ``load_model`` for an in-memory ``{hf_name: tensor}`` dict."""
     packed = getattr(model, "packed_modules_mapping", {})
     for name, tensor in state.items():
         load_tensor(model, packed, name, tensor)
+    finish_load(model)
 
 
 def random_init_(model: nn.Module, seed: int = 0, std: float = 0.02, device_fill: bool = False):
