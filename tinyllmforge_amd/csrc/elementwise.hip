@@ -288,15 +288,24 @@ __global__ __launch_bounds__(256) void argmax_partial_kernel(
   }
 }
 
-__global__ __launch_bounds__(64) void argmax_final_kernel(
+// One workgroup of THREADS (64 or 256) per row.
+template <int THREADS>
+__global__ __launch_bounds__(THREADS) void argmax_final_kernel(
     const unsigned long long *__restrict__ partial, int32_t nchunks, int64_t *__restrict__ out) {
   const int row = blockIdx.x;
   unsigned long long best = 0;
-  for (int c = threadIdx.x; c < nchunks; c += 64) {
+  for (int c = threadIdx.x; c < nchunks; c += THREADS) {
     const unsigned long long k = partial[static_cast<int64_t>(row) * nchunks + c];
     best = k > best ? k : best;
   }
   best = wave_max_u64(best);
+  if (THREADS > 64) {
+    __shared__ unsigned long long part[THREADS / 64];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = best;
+    __syncthreads();
+    if (threadIdx.x == 0)
+      for (int w = 1; w < THREADS / 64; ++w) best = part[w] > best ? part[w] : best;
+  }
   if (threadIdx.x == 0) out[row] = static_cast<int64_t>(0xffffffffu - static_cast<unsigned int>(best));
 }
 
@@ -395,7 +404,10 @@ __global__ __launch_bounds__(256) void sample_partial_kernel(
 // Last stage of the greedy sample on its own: rows x nparts keys (argmax_key) -> token ids.
 int launch_argmax_final(const unsigned long long *keys, int32_t nparts, int64_t *out, int32_t rows,
                         hipStream_t stream) {
-  hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(64), 0, stream, keys, nparts, out);
+  if (nparts > 256)  // the keys of an LM-head epilogue: thousands per row
+    hipLaunchKernelGGL(argmax_final_kernel<256>, dim3(rows), dim3(256), 0, stream, keys, nparts, out);
+  else
+    hipLaunchKernelGGL(argmax_final_kernel<64>, dim3(rows), dim3(64), 0, stream, keys, nparts, out);
   return launch_status();
 }
 
@@ -548,7 +560,7 @@ extern "C" int tlf_argmax(const void *logits, int64_t row_stride, int64_t *out, 
   hipLaunchKernelGGL(argmax_partial_kernel, dim3(nchunks, rows), dim3(256), 0,
                      static_cast<hipStream_t>(stream),
                      static_cast<const unsigned short *>(logits), row_stride, vocab, part, nchunks);
-  hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(64), 0,
+  hipLaunchKernelGGL(argmax_final_kernel<64>, dim3(rows), dim3(64), 0,
                      static_cast<hipStream_t>(stream), part, nchunks, out);
   return launch_status();
 }
@@ -570,7 +582,7 @@ extern "C" int tlf_sample(const void *logits, int64_t row_stride, const float *t
                      row_stride, vocab, temperatures, static_cast<unsigned int>(seed),
                      static_cast<unsigned int>(seed >> 32), static_cast<unsigned int>(offset),
                      static_cast<unsigned int>(offset >> 32), part, nchunks);
-  hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(64), 0,
+  hipLaunchKernelGGL(argmax_final_kernel<64>, dim3(rows), dim3(64), 0,
                      static_cast<hipStream_t>(stream), part, nchunks, out);
   return launch_status();
 }
