@@ -839,14 +839,25 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
   } else if (M <= 64) {
     // one M-tile and a very wide N (the LM head at small batch): pure weight streaming
     g.bn = 128; g.bm = 64; g.stages = 2; g.occ = 3;
-  } else if (tiles(128, 128) < 1024) {
-    g.bn = 128; g.bm = 128; g.stages = 3; g.occ = 2;
-  } else if (w8 && K >= 8192) {
-    // long K (down projections): the square tile moves the fewest bytes per flop (measured 5-6 %
-    // faster than 256 x 128 on 4096 x 12288 and 5120 x 25600)
-    g.bn = 256; g.bm = 256; g.stages = 3; g.occ = 1;
   } else if (w8) {
-    g.bn = 256; g.bm = 128; g.stages = 2; g.occ = 2;  // 64 KB of LDS: two workgroups per CU
+    // int8 weights: every wave of a tile spans all of its tokens (waves side by side along N), so
+    // each weight is converted to bf16 by one wave only; a 2 x 2 wave layout converts it twice and
+    // is 5-10 % slower although it reads fewer LDS bytes per MFMA.
+    const int t256 = tiles(256, 256);
+    const int m256 = (M + 255) / 256 * 256;  // rows the 256-token tiles would compute
+    if (t256 >= 192 && !(t256 > 256 && t256 < 512) && m256 * 20 <= M * 23) {
+      // 256 x 256 tile, eight waves of 32 channels x 256 tokens, one workgroup per CU: fewest
+      // copied bytes per flop (1.19-1.31 PFLOP/s at M = 8192 against 1.09-1.16 for 256 x 128).
+      // Between one and two tiles per CU the second round would be half empty; more than 15 % of
+      // padding rows costs more than the tile saves.
+      g.bn = 256; g.bm = 256; g.stages = 3; g.occ = 2; g.wn = 8;
+    } else if (tiles(128, 128) < 1024) {
+      g.bn = 128; g.bm = 128; g.stages = 3; g.occ = 2; g.wn = 4;
+    } else {
+      g.bn = 256; g.bm = 128; g.stages = 2; g.occ = 2; g.wn = 4;  // 64 KB of LDS: two workgroups per CU
+    }
+  } else if (tiles(128, 128) < 1024) {
+    g.bn = 128; g.bm = 128; g.stages = 3; g.occ = 2; g.wn = 2;
   } else {
     g.bn = 256; g.bm = 128; g.stages = 3; g.occ = 1;
   }
@@ -989,8 +1000,10 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
     TLF_TILE_KG(64, 128, 2, 1, 3, 2, 2)
     TLF_TILE_KG(64, 160, 2, 1, 3, 2, 2)
     TLF_TILE_KG(64, 64, 2, 2, 3, 4, 4)
+    TLF_TILE(256, 256, 8, 1, 3, 2)   // eight waves of 32 channels x 256 tokens
     TLF_TILE(256, 256, 2, 2, 3, 1)
   }
+  TLF_TILE(256, 128, 4, 1, 2, 2)
   // ... and alternatives kept for tuning through TLF_GEMM_PLAN
   TLF_TILE(128, 256, 2, 2, 2, 2)
   TLF_TILE(128, 128, 2, 2, 2, 3)
