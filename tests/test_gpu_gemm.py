@@ -49,6 +49,8 @@ SHAPES = [  # (M, N, K)
     (130, 16400, 256), (70, 16384, 192), (224, 16384, 128),
     # one M-tile, 64 channels, two wave sets splitting K (decode-size batch, moderate N)
     (150, 1024, 12288), (140, 6144, 4096), (90, 1040, 8320),
+    # 256 x 256 tile with eight waves (ragged M and N) and the 256 x 128 tile with four waves side by side
+    (2000, 24592, 192), (2050, 8208, 320), (1000, 6160, 192),
 ]
 
 
@@ -99,7 +101,7 @@ def test_bf16_gemm(M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(1, 6144, 1024), (16, 2048, 4096), (130, 24576, 1024), (300, 6144, 2048),
-                                   (2048, 4096, 512), (70, 16384, 192), (33, 272, 64)])
+                                   (2048, 4096, 512), (70, 16384, 192), (33, 272, 64), (2100, 24576, 128)])
 def test_w8a16_gemm_fused_silu_mul_equals_the_two_kernels(M, N, K):
     """gate_up projection + SiLU-and-mul in one kernel (interleaved weight rows) is bit-identical to the
     plain GEMM on the same weight followed by the activation kernel, and within tolerance of the oracle."""

@@ -856,9 +856,9 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
     } else {
       g.bn = 256; g.bm = 128; g.stages = 2; g.occ = 2; g.wn = 4;  // 64 KB of LDS: two workgroups per CU
     }
-  } else if (tiles(128, 128) < 1024) {
+  } else if (tiles(128, 128) < 1024 && tiles(256, 128) < 256) {
     g.bn = 128; g.bm = 128; g.stages = 3; g.occ = 2; g.wn = 2;
-  } else {
+  } else {  // bf16, one 256 x 128 tile per CU or more (measured 7-10 % faster than 128 x 128 from there on)
     g.bn = 256; g.bm = 128; g.stages = 3; g.occ = 1;
   }
   // a long K wants a split of its own: no workgroup walks more than ~48 K-tiles when splitting
