@@ -845,7 +845,7 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
     // is 5-10 % slower although it reads fewer LDS bytes per MFMA.
     const int t256 = tiles(256, 256);
     const int m256 = (M + 255) / 256 * 256;  // rows the 256-token tiles would compute
-    if (t256 >= 192 && !(t256 > 256 && t256 < 512) && m256 * 20 <= M * 23) {
+    if (t256 >= 160 && !(t256 > 256 && t256 < 512) && m256 * 20 <= M * 23) {
       // 256 x 256 tile, eight waves of 32 channels x 256 tokens, one workgroup per CU: fewest
       // copied bytes per flop (1.19-1.31 PFLOP/s at M = 8192 against 1.09-1.16 for 256 x 128).
       // Between one and two tiles per CU the second round would be half empty; more than 15 % of
@@ -981,15 +981,15 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
     launched = true;                                                                        \
   }
 #define TLF_TILE(BN_, BM_, WN_, WM_, NS_, OCC_) TLF_TILE_KG(BN_, BM_, WN_, WM_, NS_, OCC_, 1)
-  // the instances plan_gemm() uses ...
+  // the instances plan_gemm() uses (TLF_GEMM_PLAN can only pick among these)
   TLF_TILE(64, 64, 2, 2, 2, 4)
   TLF_TILE_KG(64, 64, 2, 2, 2, 4, 2)
   TLF_TILE_KG(64, 64, 2, 2, 2, 4, 4)
   TLF_TILE(128, 64, 4, 1, 2, 3)
   TLF_TILE(128, 64, 4, 1, 4, 3)
   TLF_TILE(128, 128, 2, 2, 3, 2)
-  TLF_TILE(256, 128, 2, 2, 2, 2)
   TLF_TILE(256, 128, 2, 2, 3, 1)
+  TLF_TILE(256, 128, 4, 1, 2, 2)
   TLF_TILE(128, 96, 4, 1, 3, 2)   // one M-tile of 96 ... 224 tokens, waves side by side along N
   TLF_TILE(128, 128, 4, 1, 3, 2)
   TLF_TILE(128, 160, 4, 1, 3, 2)
@@ -1001,13 +1001,7 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
     TLF_TILE_KG(64, 160, 2, 1, 3, 2, 2)
     TLF_TILE_KG(64, 64, 2, 2, 3, 4, 4)
     TLF_TILE(256, 256, 8, 1, 3, 2)   // eight waves of 32 channels x 256 tokens
-    TLF_TILE(256, 256, 2, 2, 3, 1)
   }
-  TLF_TILE(256, 128, 4, 1, 2, 2)
-  // ... and alternatives kept for tuning through TLF_GEMM_PLAN
-  TLF_TILE(128, 256, 2, 2, 2, 2)
-  TLF_TILE(128, 128, 2, 2, 2, 3)
-  TLF_TILE(256, 64, 4, 1, 2, 3)
 #undef TLF_TILE
 #undef TLF_TILE_KG
   if (dry) {
