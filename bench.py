@@ -237,6 +237,32 @@ def bench_gemm(args, ms=(1, 16, 64, 256, 2048, 8192)):
     return rows
 
 
+def cpu_baseline_gemm(budget_s=20.0):
+    """CPU oracle (``oracle.ops.w8a16_linear``: fp64 contraction of bf16 activations with int8 weights, scale,
+    one rounding) on the qkv projection shape at M = 256, then 2048 while the budget lasts."""
+    import torch
+    from oracle import ops as O
+    torch.manual_seed(0)
+    N, K = GEMM_SHAPES["qkv"]
+    wq = torch.randint(-127, 128, (N, K), dtype=torch.int8)
+    scale = torch.rand(N) * 9e-3 + 1e-3
+    flops, spent, done = 0.0, 0.0, []
+    for M in (256, 2048):
+        x = torch.randn(M, K).to(torch.bfloat16)
+        O.w8a16_linear(x[:16], wq, scale)                     # warm-up
+        for _ in range(3):
+            if spent >= budget_s:
+                break
+            t0 = time.perf_counter()
+            O.w8a16_linear(x, wq, scale)
+            spent += time.perf_counter() - t0
+            flops += 2.0 * M * N * K
+            done.append(M)
+    return dict(value=round(flops / spent / 1e12, 4), unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"qkv projection (N={N}, K={K}) at M = {sorted(set(done))}, {len(done)} calls, "
+                       f"{spent:.1f} s of CPU oracle time")
+
+
 # ----------------------------------------------------------------------------- config 5 (32B shape, fp8 KV, shared prefixes)
 def bench_c5(args):
     """BASELINE.json configs[4]: Qwen3-32B-shaped decoder, W8A16 linears, e4m3 KV cache with per-head scales,
@@ -407,7 +433,8 @@ def main():
             "dtype": "bf16", "data": "synthetic",
             "config": {"workload": "BASELINE.json configs[2]: y = x W^T, int8 per-channel weights, bf16 activations, the four "
                                    "Qwen3-8B projection shapes, M = 1 ... 8192, random normal x, random int8 W"},
-            "roofline": roofline, "cpu_baseline": None, "extra": extra}))
+            "roofline": roofline, "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline_gemm(),
+            "extra": extra}))
         return
     if args.workload == "decode_attn":
         cpu = None if args.no_cpu_baseline else cpu_baseline_decode(attn["case"])
