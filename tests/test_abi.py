@@ -51,6 +51,22 @@ def test_argument_rejection_happens_before_any_launch():
     assert lib.tlf_paged_decode_attn(16, 4096, 16, 16, 0, None, None, 16, 16, 16, 16,
                                      2, 32, 8, 64, 256, 16, 10, 0.1, None, 0, None) == -5  # Dh != 128
     assert lib.tlf_argmax_workspace_bytes(4, 151936) > 0
+    # the fused entry points: NULL operands, a missing or misaligned workspace, bad shapes
+    a = 4096                                                          # any 256-byte aligned non-NULL value
+    assert lib.tlf_w8a16_gemm_add_rmsnorm(a, 4096, a, a, None, a, a, a, 8, 4096, 4096, 1e-6, a, 1 << 30, None) == -1
+    assert lib.tlf_w8a16_gemm_add_rmsnorm(a, 4096, a, a, a, a, a, a, 8, 4096, 4096, 1e-6, None, 0, None) == -4
+    assert lib.tlf_w8a16_gemm_add_rmsnorm(a, 4096, a, a, a, a, a, a, 8, 32768, 4096, 1e-6, a, 1 << 30, None) == -2
+    assert lib.tlf_bf16_gemm_add_rmsnorm(a, 4096, a, a, a, a, a, 0, 4096, 4096, 1e-6, None, 0, None) == 0   # no tokens
+    assert lib.tlf_bf16_gemm_argmax(a, 4096, a, None, 8, 4096, 4096, a, 1 << 30, None) == -1
+    assert lib.tlf_bf16_gemm_argmax(a, 4096, a, a, 8, 4096, 4096, a, 16, None) == -4
+    assert lib.tlf_bf16_gemm_argmax(a, 4000, a, a, 8, 4096, 4096, a, 1 << 30, None) == -2        # row stride < K
+    assert lib.tlf_sample(a, 1024, None, a, 4, 1024, 0, 0, a, 1 << 20, None) == -1
+    assert lib.tlf_sample(a, 1000, a, a, 4, 1024, 0, 0, a, 1 << 20, None) == -2
+    assert lib.tlf_sample(a, 1024, a, a, 4, 1024, 0, 0, a, 8, None) == -4
+    m, n, k = 200, 4096, 12288
+    assert lib.tlf_gemm_add_rmsnorm_workspace_bytes(m, n, k) >= lib.tlf_w8a16_gemm_workspace_bytes(m, n, k) + m * n * 2
+    assert lib.tlf_gemm_argmax_workspace_bytes(256, 151936, 4096) >= 256 * (151936 // 32) * 8
+    assert lib.tlf_gemm_argmax_workspace_bytes(4, 151936, 4096) >= 4 * 151936 * 2 + lib.tlf_argmax_workspace_bytes(4, 151936)
 
 
 def test_ops_refuse_cpu_tensors():

@@ -124,7 +124,8 @@ def test_w8a16_gemm_fused_silu_mul_equals_the_two_kernels(M, N, K):
     (120, 4096, 4096, True, "fused"), (160, 4096, 12288, True, "fused"), (97, 1024, 3072, True, "fused"),
     (120, 4096, 4096, False, "fused"), (70, 8704, 8192, True, "fused"), (50, 256, 8192, True, "fused"),
     (40, 128, 4096, True, "fused"),
-    (256, 4096, 4096, True, "staged"), (4, 4096, 1024, True, "staged"), (2048, 1024, 3072, False, "staged")])
+    (256, 4096, 4096, True, "staged"), (4, 4096, 1024, True, "staged"), (2048, 1024, 3072, False, "staged"),
+    (32, 5120, 8192, True, "fused"), (33, 5120, 25600, True, "fused")])
 def test_row_projection_with_add_rmsnorm_equals_the_two_kernels(M, N, K, w8, path):
     """o_proj / down_proj together with the add-RMSNorm that follows: bit-identical to the GEMM entry point
     followed by tlf_add_rmsnorm on both routes -- the fused split-K reduce + norm kernel ("fused", one case
