@@ -77,6 +77,25 @@ def test_w8a16_bit_exact_on_integer_activations(M, N, K):
     assert torch.equal(got.view(torch.int16), ref.view(torch.int16))
 
 
+@pytest.mark.parametrize("M,N,K", [(8192, 6144, 4096), (8192, 4096, 12288), (2048, 24576, 4096), (16384, 4096, 4096),
+                                   (130, 24576, 4096), (256, 4096, 12288)])
+def test_w8a16_full_size_exact_on_integer_data(M, N, K):
+    """The projection shapes of the 8B configuration at prefill and decode sizes, on data whose products are
+    exact at every step: activations in {-2 .. 2}, weights in [-127, 127], scale 2^-12.  Partial sums stay
+    below 2^24, so fp32 accumulation in any order is exact and so is the one rounding to bf16 of the exact
+    result: the kernel must reproduce ``bf16(x W^T 2^-12)`` from an fp64 product bit for bit.  (The CPU oracle
+    takes minutes at these sizes; the fp64 product is its definition, evaluated on the device.)"""
+    from tinyllmforge_amd import ops as P
+    x = torch.randint(-2, 3, (M, K), generator=g(M), dtype=torch.int32).to(BF).to(DEV)
+    wq = torch.randint(-127, 128, (N, K), generator=g(N + K), dtype=torch.int32).to(torch.int8).to(DEV)
+    scale = torch.full((N,), 2.0 ** -12, device=DEV)
+    got = P.w8a16_linear(x, wq, scale)
+    for m0 in range(0, M, 2048):                          # fp64 reference in slabs of 2048 tokens
+        ref = (x[m0:m0 + 2048].double() @ wq.double().t()) * 2.0 ** -12
+        assert torch.equal(got[m0:m0 + 2048].view(torch.int16), ref.to(BF).view(torch.int16)), m0
+    assert (got.float().abs().max() > 0.05)               # not a vacuous comparison
+
+
 def test_w8a16_strided_activations_and_3d_input():
     from tinyllmforge_amd import ops as P
     M, N, K = 40, 1024, 1024
