@@ -1073,9 +1073,18 @@ using namespace tlf;
 
 extern "C" size_t tlf_w8a16_gemm_workspace_bytes(int32_t M, int32_t N, int32_t K) {
   if (M <= 0 || N <= 0 || K <= 0 || K % kBK) return 0;
-  // room for the deepest split any plan may use (16), so that tuning overrides stay in bounds
   if (M <= skinny_max_m()) return 0;
-  return static_cast<size_t>(16) * M * N * sizeof(float);
+  // fp32 partial sums of the plan's split of K (the larger of the int8 and the bf16 plan: both
+  // entry points share this query); a tuning override may pick any split up to 16
+  int splits = 16;
+  if (!getenv("TLF_GEMM_PLAN")) {
+    int32_t p8[8], p16[8];
+    if (launch_gemm<true>(nullptr, K, nullptr, nullptr, nullptr, M, N, K, nullptr, 0, nullptr, p8) == TLF_OK &&
+        launch_gemm<false>(nullptr, K, nullptr, nullptr, nullptr, M, N, K, nullptr, 0, nullptr, p16) == TLF_OK)
+      splits = p8[5] > p16[5] ? p8[5] : p16[5];
+  }
+  if (splits <= 1) return 0;
+  return static_cast<size_t>(splits) * M * N * sizeof(float);
 }
 
 extern "C" int tlf_w8a16_gemm(const void *x, int64_t x_stride, const void *wq, const float *scale,
