@@ -192,6 +192,9 @@ int tlf_sample(const void *logits, int64_t row_stride, const float *temperatures
  *
  * x: bf16 [M, K] row stride x_stride (elements); wq: int8 [N, K] contiguous;
  * scale: fp32 [N]; y: bf16 [M, N] contiguous.  K % 64 == 0, N % 16 == 0.
+ * workspace: fp32 partial sums when the kernel plan for (M, N, K) splits K across workgroups
+ * (few output tiles, long K); tlf_w8a16_gemm_workspace_bytes gives the size for this and for
+ * tlf_bf16_gemm (0 when neither plan splits), 16-byte aligned.
  */
 size_t tlf_w8a16_gemm_workspace_bytes(int32_t M, int32_t N, int32_t K);
 int tlf_w8a16_gemm(const void *x, int64_t x_stride, const void *wq, const float *scale,
