@@ -389,7 +389,7 @@ def decode_byte_floor(hf, st, quantization, kv_itemsize):
                 frac=round(floor_s / max(st["decode_time"], 1e-9), 4))
 
 
-def cpu_baseline_e2e(llm, prompts, nseq=2, out_tokens=4):
+def cpu_baseline_e2e(llm, prompts, nseq=3, out_tokens=6):
     """CPU oracle (bf16 F.linear, the reference's own CPU arithmetic) on the first ``nseq`` sequences of the
     same workload, ``out_tokens`` greedy tokens each, with the same weights copied from the GPU model."""
     import torch
