@@ -25,41 +25,46 @@ class Scheduler:
         self.waiting.append(seq)
 
     def schedule(self) -> tuple[list[Sequence], bool]:
-        batch: list[Sequence] = []
-        budget_used = 0
-        # prefill has priority; admission looks at the full length, the budget is charged the
-        # uncached part (scheduler.py:29,33)
-        while self.waiting and len(batch) < self.max_num_seqs:
-            seq = self.waiting[0]
-            if budget_used + len(seq) > self.max_num_batched_tokens or not self.block_manager.can_allocate(seq):
-                break
-            self.block_manager.allocate(seq)
-            budget_used += len(seq) - seq.num_cached_tokens
-            seq.status = SequenceStatus.RUNNING
-            self.waiting.popleft()
-            self.running.append(seq)
-            batch.append(seq)
-        if batch:
-            return batch, True
+        """The next step's sequences and whether it is a prefill step.  Prefill has priority: a step
+        never mixes the two kinds (scheduler.py:22-57)."""
+        admitted = self._admit_waiting()
+        if admitted:
+            return admitted, True
+        return self._step_running(), False
 
-        # decode: every running sequence gets one token; when no block is left, the newest
-        # running sequence is preempted (freed and put back at the head of the waiting queue)
+    def _admit_waiting(self) -> list[Sequence]:
+        # admission looks at the full length, the budget is charged the uncached part (scheduler.py:29,33)
+        batch: list[Sequence] = []
+        charged = 0
+        while self.waiting and len(batch) < self.max_num_seqs:
+            head = self.waiting[0]
+            fits = charged + len(head) <= self.max_num_batched_tokens and self.block_manager.can_allocate(head)
+            if not fits:
+                break
+            self.block_manager.allocate(head)
+            charged += len(head) - head.num_cached_tokens
+            head.status = SequenceStatus.RUNNING
+            self.running.append(self.waiting.popleft())
+            batch.append(head)
+        return batch
+
+    def _step_running(self) -> list[Sequence]:
+        # every running sequence gets one token; when no block is left for one of them, the newest
+        # running sequence is preempted (freed, back to the head of the waiting queue) until it fits,
+        # the sequence itself if it is the last one left
+        batch: list[Sequence] = []
         while self.running and len(batch) < self.max_num_seqs:
             seq = self.running.popleft()
-            evicted_self = False
-            while not self.block_manager.can_append(seq):
-                if self.running:
-                    self.preempt(self.running.pop())
-                else:
-                    self.preempt(seq)
-                    evicted_self = True
-                    break
-            if not evicted_self:
+            while not self.block_manager.can_append(seq) and self.running:
+                self.preempt(self.running.pop())
+            if self.block_manager.can_append(seq):
                 self.block_manager.may_append(seq)
                 batch.append(seq)
+            else:
+                self.preempt(seq)
         assert batch
         self.running.extendleft(reversed(batch))
-        return batch, False
+        return batch
 
     def preempt(self, seq: Sequence):
         seq.status = SequenceStatus.WAITING

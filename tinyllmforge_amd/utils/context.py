@@ -1,41 +1,61 @@
 """Attention metadata side channel (reference: tinyvllm/utils/context.py:5-27).
 
-``Attention`` and ``ParallelLMHead`` read the step's metadata from a module-level
-``Context`` that the model runner sets before each forward pass.
+``Attention`` and ``ParallelLMHead`` do not take the step's metadata as arguments: the model runner
+publishes it here before each forward pass and the layers read it back, which keeps the layer
+signatures those of the reference.  One ``Context`` object lives for the whole process and is
+rewritten in place (a decode step publishes three tensors a thousand times per request batch;
+nothing is allocated for that), so a caller must not hold on to ``get_context()`` across steps.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass
+# field -> value after reset_context(); the order is the positional order of set_context()
+_FIELDS = (
+    ("is_prefill", False),      # prefill or decode step
+    ("cu_seqlens_q", None),     # prefill: int32 [B + 1] prefix sums of the query lengths
+    ("cu_seqlens_k", None),     # prefill: the same for the key lengths (cached prefix included)
+    ("max_seqlen_q", 0),        # prefill
+    ("max_seqlen_k", 0),        # prefill
+    ("slot_mapping", None),     # both: int32 [N] cache slot of every token of the step
+    ("context_lens", None),     # decode: int32 [B] tokens per sequence, the new one included
+    ("block_tables", None),     # decode, and prefill with a prefix hit: int32 [B, max blocks]
+)
 
-import torch
 
-
-@dataclass
 class Context:
-    is_prefill: bool = False
-    cu_seqlens_q: torch.Tensor | None = None
-    cu_seqlens_k: torch.Tensor | None = None
-    max_seqlen_q: int = 0
-    max_seqlen_k: int = 0
-    slot_mapping: torch.Tensor | None = None
-    context_lens: torch.Tensor | None = None
-    block_tables: torch.Tensor | None = None
+    __slots__ = tuple(name for name, _ in _FIELDS)
+
+    def __init__(self):
+        self.clear()
+
+    def clear(self):
+        for name, default in _FIELDS:
+            setattr(self, name, default)
+
+    def __repr__(self):
+        return "Context(" + ", ".join(f"{n}={getattr(self, n)!r}" for n, _ in _FIELDS) + ")"
 
 
-_CONTEXT = Context()
+_CURRENT = Context()
 
 
 def get_context() -> Context:
-    return _CONTEXT
+    return _CURRENT
 
 
-def set_context(is_prefill, cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=0, max_seqlen_k=0,
-                slot_mapping=None, context_lens=None, block_tables=None):
-    global _CONTEXT
-    _CONTEXT = Context(is_prefill, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-                       slot_mapping, context_lens, block_tables)
+def set_context(is_prefill, *values, **named):
+    """``set_context(is_prefill, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, slot_mapping,
+    context_lens, block_tables)``, every argument after the first optional, positional or by name."""
+    _CURRENT.clear()
+    _CURRENT.is_prefill = is_prefill
+    if len(values) > len(_FIELDS) - 1:
+        raise TypeError(f"set_context takes at most {len(_FIELDS)} positional arguments")
+    for (name, _), value in zip(_FIELDS[1:], values):
+        setattr(_CURRENT, name, value)
+    for name, value in named.items():
+        if name not in Context.__slots__ or name == "is_prefill":
+            raise TypeError(f"set_context got an unexpected argument {name!r}")
+        setattr(_CURRENT, name, value)
 
 
 def reset_context():
-    global _CONTEXT
-    _CONTEXT = Context()
+    _CURRENT.clear()
