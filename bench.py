@@ -12,9 +12,10 @@ beside it) on the reference's own bench.py recipe (tinyvllm bench.py:39-59): ``s
 prompts of ``randint(100, 1024)`` random token ids, ``max_tokens = randint(100, 1024)``,
 ``ignore_eos``, continuous batching, hipGraph-captured decode, one warm-up ``generate`` first;
 tok/s = sum(max_tokens) / wall time of ``generate()``, prefill included.  Greedy sampling
-(temperature 0; the reference's script uses 0.6) keeps the run deterministic.  A "step" is one
-engine step (one prefill or one decode pass over the running batch); ``--steps K`` stops the
-timed run after K engine steps (0 = the whole job).
+(temperature 0; the reference's script uses 0.6, timed as a second leg) keeps the run
+deterministic.  A "step" is one engine step (one prefill or one decode pass over the running
+batch).  ``value`` is always the whole job; ``--steps K`` only chooses what ``steps`` and
+``ms_per_step`` describe: the first K engine steps of that same timed run (0 = all of them).
 
 ``roofline`` is the paged decode attention kernel, the largest single consumer of a decode step,
 measured live with HIP events on its launch stream on BASELINE.json configs[1]
@@ -48,7 +49,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=0, help="timed engine steps of the e2e run (0 = whole job)")
+    ap.add_argument("--steps", type=int, default=0,
+                    help="engine steps that steps/ms_per_step describe (0 = all); value is always the whole job")
     ap.add_argument("--warmup", type=int, default=1, help="warm-up generate() calls before the timed run")
     ap.add_argument("--workload", default="e2e", choices=["e2e", "decode_attn", "gemm", "c5", "all"])
     ap.add_argument("--attn-steps", type=int, default=200, help="timed launches of the decode-attention microbench")
@@ -56,6 +58,8 @@ def parse():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--skip-bf16", action="store_true", help="e2e: skip the second run with bf16 linears (profiling)")
+    ap.add_argument("--skip-c5", action="store_true", help="e2e: skip the Qwen3-32B-shape run (configs[4])")
+    ap.add_argument("--skip-gemm", action="store_true", help="e2e: skip the W8A16 GEMM table (configs[2])")
     return ap.parse_args()
 
 
@@ -216,24 +220,38 @@ def cpu_baseline_decode(case, budget_s=20.0):
 GEMM_SHAPES = {"qkv": (6144, 4096), "o_proj": (4096, 4096), "gate_up": (24576, 4096), "down": (4096, 12288)}
 
 
-def bench_gemm(args, ms=(1, 16, 64, 256, 2048, 8192)):
+def bench_gemm(args, ms=(1, 16, 64, 128, 256, 2048, 8192)):
+    """W8A16 GEMM table.  Up to M = 256 a decode step finds its weights in HBM (a layer's weights were last
+    touched one whole step ago), so those cells cycle through enough copies of the weight to exceed the
+    256 MB Infinity Cache several times ("cold"); the same call on one resident copy is reported beside it
+    ("warm").  Larger M is compute bound and timed on one copy."""
     import torch
     from tinyllmforge_amd import ops as P
     torch.manual_seed(0)
     rows = []
     for name, (N, K) in GEMM_SHAPES.items():
-        wq = torch.randint(-127, 128, (N, K), device="cuda", dtype=torch.int8)
+        copies = max(2, -(-(768 << 20) // (N * K)))
+        wqs = [torch.randint(-127, 128, (N, K), device="cuda", dtype=torch.int8) for _ in range(copies)]
         scale = torch.rand(N, device="cuda") * 9e-3 + 1e-3
         for M in ms:
             x = torch.randn(M, K, device="cuda").to(torch.bfloat16)
-            sec = time_graph(lambda: P.w8a16_linear(x, wq, scale)) * 1e-3
+            warm = time_graph(lambda: P.w8a16_linear(x, wqs[0], scale)) * 1e-3
+            sec = warm
+            if M <= 256:
+                def cycle():
+                    for w in wqs:
+                        P.w8a16_linear(x, w, scale)
+                sec = time_graph(cycle, launches=2, replays=10) * 1e-3 / copies
             nbytes = N * K + 4 * N + 2 * M * K + 2 * M * N
             flops = 2.0 * M * N * K
-            bound = "hbm" if M <= 64 else "mfma"
-            rows.append(dict(shape=name, M=M, N=N, K=K, us=round(sec * 1e6, 2), GBps=round(nbytes / sec / 1e9, 1),
+            bound = "hbm" if M <= 128 else "mfma"
+            rows.append(dict(shape=name, M=M, N=N, K=K, us=round(sec * 1e6, 2), weights="cold" if M <= 256 else "warm",
+                             us_warm=round(warm * 1e6, 2), GBps=round(nbytes / sec / 1e9, 1),
                              TFLOPs=round(flops / sec / 1e12, 1), bound=bound,
                              frac=round((nbytes / sec / 1e9 / HBM_PEAK_GBPS) if bound == "hbm"
                                         else (flops / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS), 4)))
+        del wqs
+        torch.cuda.empty_cache()
     return rows
 
 
@@ -309,6 +327,34 @@ def e2e_workload(num_seqs=256):
     return prompts, max_tokens
 
 
+def timed_generate(llm, prompts, sps, mark_steps=0):
+    """The engine's generate() loop (tinyvllm llm_engine.py:64-101) with its per-step statistics, plus the
+    wall time at which the first ``mark_steps`` engine steps were done.  Returns (stats, wall_s, wall_at_mark)."""
+    import torch
+    for p, sp in zip(prompts, sps):
+        llm.add_request(p, sp)
+    st = dict(prefill_steps=0, decode_steps=0, prefill_time=0.0, decode_time=0.0, cached_prompt_tokens=0,
+              decode_context_tokens=0)
+    steps, at_mark = 0, None
+    torch.cuda.synchronize()
+    t_begin = time.perf_counter()
+    while not llm.is_finished():
+        t0 = time.perf_counter()
+        _, num_tokens = llm.step()            # ends in the step's device -> host copy of the token ids
+        dt = time.perf_counter() - t0
+        kind = "prefill" if num_tokens > 0 else "decode"
+        st[kind + "_steps"] += 1
+        st[kind + "_time"] += dt
+        st["cached_prompt_tokens"] += llm._step_info[0]
+        st["decode_context_tokens"] += llm._step_info[1]
+        steps += 1
+        if steps == mark_steps:
+            at_mark = time.perf_counter() - t_begin
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t_begin
+    return st, wall, at_mark
+
+
 def bench_e2e(args, quantization):
     import torch
     from tinyllmforge_amd import LLM, SamplingParams
@@ -320,50 +366,27 @@ def bench_e2e(args, quantization):
     sps = [SamplingParams(temperature=0.0, ignore_eos=True, max_tokens=m) for m in max_tokens]
     for _ in range(max(1, args.warmup)):
         llm.generate([[1, 2, 3, 4, 5, 6, 7, 8]], SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    if args.steps > 0:                       # a bounded number of engine steps
-        for p, sp in zip(prompts, sps):
-            llm.add_request(p, sp)
-        produced, steps = 0, 0
-        while not llm.is_finished() and steps < args.steps:
-            seqs, is_prefill = llm.scheduler.schedule()
-            toks = llm.model_runner.call("run", seqs, is_prefill)
-            llm.scheduler.postprocess(seqs, toks)
-            produced += len(seqs)          # every scheduled sequence gains one token, prefill or decode
-            steps += 1
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        total, stats = produced, dict(steps=steps)
-        # drain what is left so that the engine can be torn down cleanly
-        while not llm.is_finished():
-            llm.step()
+    st, wall, at_mark = timed_generate(llm, prompts, sps, args.steps)
+    total = sum(max_tokens)                  # every sequence runs to its max_tokens (ignore_eos)
+    all_steps = st["prefill_steps"] + st["decode_steps"]
+    stats = dict(steps=all_steps, prefill_steps=st["prefill_steps"], decode_steps=st["decode_steps"],
+                 prefill_s=round(st["prefill_time"], 3), decode_s=round(st["decode_time"], 3),
+                 decode_ms_per_step=round(1e3 * st["decode_time"] / max(1, st["decode_steps"]), 3),
+                 decode_byte_floor=decode_byte_floor(llm.config.hf_config, st, quantization, kv_itemsize=2))
+    if args.steps > 0 and at_mark is not None:
+        slice_steps, slice_s = args.steps, at_mark
     else:
-        llm.generate(prompts, sps)
-        torch.cuda.synchronize()
-        wall = time.perf_counter() - t0
-        total = sum(max_tokens)
-        st = llm.last_stats
-        stats = dict(steps=st["prefill_steps"] + st["decode_steps"], prefill_steps=st["prefill_steps"],
-                     decode_steps=st["decode_steps"], prefill_s=round(st["prefill_time"], 3),
-                     decode_s=round(st["decode_time"], 3),
-                     decode_ms_per_step=round(1e3 * st["decode_time"] / max(1, st["decode_steps"]), 3))
-    if "decode_context_tokens" in (llm.last_stats or {}) and args.steps == 0:
-        stats["decode_byte_floor"] = decode_byte_floor(llm.config.hf_config, llm.last_stats, quantization, kv_itemsize=2)
+        slice_steps, slice_s = all_steps, wall
     res = dict(tok_s=total / wall, wall_s=wall, total_output_tokens=total, init_s=round(init_s, 1), stats=stats,
-               kv_blocks=llm.config.num_kvcache_blocks)
-    if quantization is not None and args.steps == 0:
+               kv_blocks=llm.config.num_kvcache_blocks, slice_steps=slice_steps, slice_s=slice_s)
+    if quantization is not None:
         # the reference's script samples at temperature 0.6 (bench.py:49): same workload through the
         # logits + sampling-kernel path instead of the fused LM head + argmax
         hot = [SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=m) for m in max_tokens]
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        llm.generate([[(t + 1) % 10001 for t in p] for p in prompts], hot)   # other tokens: no prefix-cache hits
-        torch.cuda.synchronize()
-        w = time.perf_counter() - t0
+        shifted = [[(t + 1) % 10001 for t in p] for p in prompts]          # other tokens: no prefix-cache hits
+        st6, w, _ = timed_generate(llm, shifted, hot)
         res["temperature_0.6"] = dict(tok_s=round(total / w, 1), wall_s=round(w, 3),
-                                      decode_ms_per_step=round(1e3 * llm.last_stats["decode_time"] /
-                                                               max(1, llm.last_stats["decode_steps"]), 3))
+                                      decode_ms_per_step=round(1e3 * st6["decode_time"] / max(1, st6["decode_steps"]), 3))
     cpu = None
     if quantization is None and not args.no_cpu_baseline:
         cpu = cpu_baseline_e2e(llm, prompts)
@@ -450,12 +473,16 @@ def main():
         return
     del attn
     torch.cuda.empty_cache()
-    if args.workload in ("c5", "all"):
-        a8 = bench_decode_attn(args, fp8=True, hq=64)   # the decode microbench on e4m3 rows, 64 query heads
-        a8.pop("case")
-        torch.cuda.empty_cache()
+    if args.workload == "e2e" and not args.skip_gemm:
+        extra["w8a16_gemm"] = bench_gemm(args)          # BASELINE.json configs[2]
+    # the decode microbench on e4m3 rows with 64 query heads (the 32B shape's attention)
+    a8 = bench_decode_attn(args, fp8=True, hq=64)
+    a8.pop("case")
+    extra["paged_decode_fp8_rows"] = a8["roofline"]
+    del a8
+    torch.cuda.empty_cache()
+    if args.workload in ("c5", "all") or (args.workload == "e2e" and not args.skip_c5):
         c5 = bench_c5(args)
-        c5["paged_decode_fp8_rows"] = a8["roofline"]
         extra["config5_qwen3_32b_fp8kv"] = c5
         import gc
         gc.collect()
@@ -482,15 +509,15 @@ def main():
                               "kv_blocks": w8["kv_blocks"]}
     if "temperature_0.6" in w8:
         extra["w8a16_linears"]["temperature_0.6"] = w8["temperature_0.6"]
-    steps = w8["stats"]["steps"]
+    whole = w8["slice_steps"] == w8["stats"]["steps"]
     out = {
         "metric": "output tok/s (Qwen3-8B-shape, 1 GPU); paged-decode HBM GB/s vs peak",
         "value": round(w8["tok_s"], 1),
         "unit": "tok/s",
         "n_gpus": 1,
-        "steps": steps,
+        "steps": w8["slice_steps"],
         "warmup": max(1, args.warmup),
-        "ms_per_step": round(1e3 * w8["wall_s"] / max(1, steps), 4),
+        "ms_per_step": round(1e3 * w8["slice_s"] / max(1, w8["slice_steps"]), 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -498,8 +525,12 @@ def main():
         "data": "synthetic",
         "config": {"workload": "BASELINE.json configs[3]: end-to-end Qwen3-8B-shaped decoder, random-init, W8A16 linears "
                                "(int8 weights, bf16 activations and MFMA), bf16 KV cache, %d sequences, prompts and outputs "
-                               "~U[100,1024] tokens, ignore_eos, greedy, continuous batching, hipGraph decode"
-                               % args.num_seqs,
+                               "~U[100,1024] tokens, ignore_eos, greedy, continuous batching, hipGraph decode; value = "
+                               "sum(max_tokens) / wall time of the WHOLE job (%d engine steps, %.3f s)"
+                               % (args.num_seqs, w8["stats"]["steps"], w8["wall_s"]),
+                   "steps_describe": ("all engine steps of the timed job" if whole else
+                                      "the first %d engine steps of the same timed job (prefill-heavy: the job starts "
+                                      "with its prefill steps); ms_per_step is their mean" % w8["slice_steps"]),
                    "total_output_tokens": w8["total_output_tokens"],
                    "roofline_workload": "BASELINE.json configs[1] paged decode attention microbench"},
         "roofline": roofline,

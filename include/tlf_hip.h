@@ -115,8 +115,8 @@ int tlf_add_rmsnorm(const void *x, const void *residual, const void *weight,
  *
  * q: [n, num_q_heads*head_dim] bf16 with row stride q_stride (elements), k
  * likewise; outputs contiguous and may alias the inputs.  positions int64 [n],
- * each in [0, max_pos) (rows with a position outside the table are left
- * untouched).  head_dim % 16 == 0.
+ * each in [0, max_pos) (a row whose position lies outside the table is copied
+ * to the output unrotated; tlf_qknorm_rope_store does the same).  head_dim % 16 == 0.
  */
 int tlf_rope(const int64_t *positions, const void *q, int64_t q_stride,
              const void *k, int64_t k_stride, const float *cos_sin,
@@ -291,8 +291,9 @@ int tlf_gemm_plan(int32_t M, int32_t N, int32_t K, int32_t w8, int32_t *plan8);
  * never dereferenced (the reference pads them with -1 or 0); entries outside
  * [0, num_cache_blocks) inside that range make the kernel skip the block.
  * context_lens int32 [batch]; a sequence with context_len <= 0 gets zeros.
- * out: bf16 [batch, Hq*Dh] contiguous.  fp32 softmax and accumulation, bf16
- * probabilities in the P.V product (as flash-attn does).
+ * out: bf16 [batch, Hq*Dh] contiguous.  fp32 softmax and accumulation; the
+ * probabilities enter the P.V product as a bf16 hi + lo pair (about 16 significant bits;
+ * flash-attn rounds them to one bf16).
  * Dh == 128, Hq % Hkv == 0, Hq/Hkv <= 16, Hkv in {1,2,4,8,16}, block_size % 16 == 0,
  * batch <= 1024.
  * Calls that share a workspace must not overlap in time.

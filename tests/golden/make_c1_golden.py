@@ -2,6 +2,7 @@
 
     python tests/golden/make_c1_golden.py            # bf16 linears, 32 tokens -> c1_greedy.json
     python tests/golden/make_c1_golden.py --w8a16    # int8 projections, 8 tokens -> c1_w8a16_greedy.json
+Beside each .json: *_hidden_bf16_bits.npy, the final hidden states (bf16 bits) behind every step's logits.
 
 Config 1: Qwen3-0.6B-shaped decoder (28 layers, hidden 1024, 16 query / 8 KV heads, head_dim 128,
 intermediate 3072, vocab 151936, RMSNorm eps 1e-6 + q/k-norm, RoPE theta 1e6, tied embeddings),
@@ -55,7 +56,8 @@ def main():
     params = c1_params(cfg)
     oracle = OracleQwen3(vars(cfg), params, w8a16=w8)
     prompts = c1_prompts()
-    ids, margins, topk = greedy_generate(oracle, prompts, max_tokens=8 if w8 else 32, block_size=256)
+    hidden = []
+    ids, margins, topk = greedy_generate(oracle, prompts, max_tokens=8 if w8 else 32, block_size=256, trace=hidden)
     out = dict(config="BASELINE.json configs[0]" + (" with int8 per-channel projection weights" if w8 else ""),
                seed=0, prompt_first_tokens=[p[:4] for p in prompts],
                token_ids=ids, top2_margin=[[round(m, 6) for m in row] for row in margins],
@@ -64,6 +66,11 @@ def main():
     path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "c1_w8a16_greedy.json" if w8 else "c1_greedy.json")
     with open(path, "w") as f:
         json.dump(out, f)
+    # the final hidden states behind every step's logits, bf16 bit patterns [steps, 4, hidden]: with the LM head
+    # weight (an input both sides share) they determine the oracle's whole logit rows
+    import numpy as np
+    bits = torch.stack(hidden).view(torch.int16).numpy()
+    np.save(path.replace("_greedy.json", "_hidden_bf16_bits.npy"), bits)
     print("wrote", path, "in %.1f s" % (time.time() - t0))
     print("min margin", min(min(r) for r in margins))
 

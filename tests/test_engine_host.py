@@ -156,6 +156,24 @@ def test_eos_stops_unless_ignored():
     assert a.is_finished and not b.is_finished
 
 
+def test_sequence_is_finished_before_its_position_leaves_the_rope_table():
+    """A decode step feeds position len(seq) (len(seq) - 1 without the reference's quirk) into a RoPE table of
+    max_position_embeddings rows: the scheduler ends a sequence whose next step would index past it."""
+    for quirk, last_len in ((True, 512), (False, 513)):
+        cfg = _cfg(model=dict(QWEN3_SHAPES["qwen3-0.6b"], max_position_embeddings=512), max_model_len=512,
+                   decode_position_quirk=quirk)
+        sch = Scheduler(cfg)
+        s = seq(508, max_tokens=100, ignore_eos=True)
+        sch.add(s)
+        positions = []
+        while not sch.is_finished():
+            batch, is_prefill = sch.schedule()
+            if not is_prefill:
+                positions.append(int(I.decode_inputs(batch, 256, quirk)["positions"][0]))
+            sch.postprocess(batch, [7])
+        assert len(s) == last_len and max(positions) == 511, (quirk, len(s), positions)
+
+
 # ----------------------------------------------------------------------------- integer inputs
 def test_prefill_inputs_closed_form_no_prefix():
     bm = BlockManager(16, BS)

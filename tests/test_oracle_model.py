@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from oracle import ops as O
-from oracle.model import OracleQwen3, greedy_generate
+from oracle.model import OracleQwen3, OracleSession, greedy_generate
 
 TINY = dict(hidden_size=256, num_hidden_layers=2, num_attention_heads=2, num_key_value_heads=1, head_dim=128,
             intermediate_size=512, vocab_size=512, max_position_embeddings=1024, rope_theta=1e6, rms_norm_eps=1e-6)
@@ -63,9 +63,9 @@ def test_decode_position_quirk_changes_the_rotation():
         c = cache()
         cu = torch.tensor([0, n], dtype=torch.int32)
         model.forward(torch.tensor(prompts[0]), torch.arange(n), c, torch.arange(n, dtype=torch.int32),
-                      lambda q, k, v, kc, vc: O.varlen_prefill_attention(q, k, v, cu, cu, 128 ** -0.5))
+                      lambda q, k, v, kc, vc, ks, vs: O.varlen_prefill_attention(q, k, v, cu, cu, 128 ** -0.5))
         h = model.forward(torch.tensor([7]), torch.tensor([pos]), c, torch.tensor([n], dtype=torch.int32),
-                          lambda q, k, v, kc, vc: O.paged_decode_attention(q, kc, vc, torch.tensor([n + 1], dtype=torch.int32), bt, 128 ** -0.5))
+                          lambda q, k, v, kc, vc, ks, vs: O.paged_decode_attention(q, kc, vc, torch.tensor([n + 1], dtype=torch.int32), bt, 128 ** -0.5))
         outs.append(h)
         # the new K row went to slot n
         assert c[0][0].view(-1, 128)[n].abs().sum() > 0 and c[0][0].view(-1, 128)[n + 1].abs().sum() == 0
@@ -108,3 +108,41 @@ def test_w8a16_oracle_routes_the_projections_through_the_int8_linear():
     _, _, t16 = greedy_generate(m16, prompts, max_tokens=1, block_size=8)
     a, b = torch.tensor(t8[0][1][0]), torch.tensor(t16[0][1][0])
     assert (a - b).abs().max() < 0.25 * b.abs().max() and not torch.equal(a, b)
+
+
+def test_session_steps_equal_the_generate_loop_and_a_cached_prefix_changes_nothing():
+    """``OracleSession`` against ``greedy_generate`` (same hidden states -> same ids), and the paged prefill with
+    a cached prefix against a dense prefill of the same prompts: with bf16 caches the prefix rows read back
+    from the cache are the bits the dense path computes, so the last-token hidden states must be equal."""
+    model = OracleQwen3(TINY, tiny_params())
+    g = torch.Generator().manual_seed(5)
+    shared = torch.randint(0, 512, (16,), generator=g).tolist()          # two full blocks of 8
+    prompts = [shared + torch.randint(0, 512, (n,), generator=g).tolist() for n in (5, 11)]
+    ids, _, _ = greedy_generate(model, prompts, max_tokens=3, block_size=8)
+    # dense: each sequence owns its blocks
+    ses = OracleSession(model, num_blocks=16, block_size=8)
+    tables = [[0, 1, 2, 3], [4, 5, 6, 7]]
+    h0 = ses.prefill(prompts, tables, [0, 0])
+    seqs = [list(p) for p in prompts]
+    got = [[] for _ in prompts]
+    h = h0
+    for step in range(3):
+        toks = O.greedy_sample(model.logits(h)).tolist()
+        for b, t in enumerate(toks):
+            seqs[b].append(t); got[b].append(t)
+        if step < 2:
+            h = ses.decode(seqs, tables)
+    assert got == ids
+    # paged: a first request fills the shared blocks 0, 1; the batch then shares them
+    ses2 = OracleSession(model, num_blocks=16, block_size=8)
+    ses2.prefill([shared + [1]], [[0, 1, 2]], [0])
+    h1 = ses2.prefill(prompts, [[0, 1, 3, 4], [0, 1, 5, 6]], [16, 16])
+    assert torch.equal(h0, h1)
+    # fp8 caches (build-defined): same driver, e4m3 rows with per-head scales; close to bf16, not equal
+    scales = [(torch.tensor([0.05]), torch.tensor([0.03]))] * TINY["num_hidden_layers"]
+    ses3 = OracleSession(model, num_blocks=16, block_size=8, kv_dtype=torch.float8_e4m3fn, kv_scales=scales)
+    ses3.prefill([shared + [1]], [[0, 1, 2]], [0])
+    h2 = ses3.prefill(prompts, [[0, 1, 3, 4], [0, 1, 5, 6]], [16, 16])
+    rel = (h2.float() - h0.float()).norm() / h0.float().norm()
+    assert 0 < rel < 0.1
+    assert ses3.caches[0][0].dtype == torch.float8_e4m3fn and ses3.caches[0][0].view(-1, 128)[0].float().abs().sum() > 0

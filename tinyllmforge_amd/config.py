@@ -78,6 +78,10 @@ class Config:
     # additions of this build (the reference has neither)
     quantization: str | None = None         # None (bf16 linears) or "w8a16"
     kv_cache_dtype: str = "bf16"            # "bf16" or "fp8_e4m3"
+    # static scales of an e4m3 cache, c = e4m3(sat(x / scale)): a float, [Hkv] values or [L][Hkv] values.
+    # 1/16 represents |x| <= 28 (448 / 16); larger K or V entries saturate.
+    kv_k_scale: Any = 1.0 / 16
+    kv_v_scale: Any = 1.0 / 16
     seed: int = 0                           # random-init seed when no weights are given
     decode_position_quirk: bool = True      # reference feeds positions = len(seq) in decode (model_runner.py:219)
 

@@ -527,7 +527,7 @@ extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void
   p.part_ml = reinterpret_cast<float *>(ws + decode_meta_bytes());
   p.part_o = p.part_ml + slots * num_q_heads * 2;
 
-  // persistent grid: two workgroups per CU, fewer when the largest possible job is small
+  // persistent grid: one workgroup per CU (decode_wgs_per_cu), fewer when the largest possible job is small
   const int64_t max_tiles = static_cast<int64_t>(batch) * ((static_cast<int64_t>(max_blocks) * block_size + kTile - 1) / kTile);
   int64_t grid = static_cast<int64_t>(decode_wgs_per_cu()) * device_cu_count();
   if (grid > kMaxGrid) grid = kMaxGrid;

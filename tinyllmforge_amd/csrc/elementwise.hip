@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) void rope_kernel(
   const int h = static_cast<int>((item / cpt) % heads);
   const int64_t tok = item / (static_cast<int64_t>(cpt) * heads);
   const int64_t pos = positions[tok];
-  if (pos < 0 || pos >= max_pos) return;
+  const bool pos_ok = pos >= 0 && pos < max_pos;  // outside the table: the row is passed through unrotated
   const bool is_q = h < num_q_heads;
   const int hh = is_q ? h : h - num_q_heads;
   const unsigned short *src = (is_q ? q + tok * q_stride : k + tok * k_stride) + hh * head_dim;
@@ -99,14 +99,14 @@ __global__ __launch_bounds__(256) void rope_kernel(
   float x1[8], x2[8];
   unpack8(*reinterpret_cast<const uint4 *>(src + c * 8), x1);
   unpack8(*reinterpret_cast<const uint4 *>(src + half + c * 8), x2);
-  const float *cs = cos_sin + pos * head_dim;
+  const float *cs = cos_sin + (pos_ok ? pos : 0) * head_dim;
   float y1[8], y2[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const float co = cs[c * 8 + i];
     const float si = cs[half + c * 8 + i];
-    y1[i] = __fsub_rn(__fmul_rn(co, x1[i]), __fmul_rn(si, x2[i]));
-    y2[i] = __fadd_rn(__fmul_rn(co, x2[i]), __fmul_rn(si, x1[i]));
+    y1[i] = pos_ok ? __fsub_rn(__fmul_rn(co, x1[i]), __fmul_rn(si, x2[i])) : x1[i];
+    y2[i] = pos_ok ? __fadd_rn(__fmul_rn(co, x2[i]), __fmul_rn(si, x1[i])) : x2[i];
   }
   *reinterpret_cast<uint4 *>(dst + c * 8) = pack8(y1);
   *reinterpret_cast<uint4 *>(dst + half + c * 8) = pack8(y2);

@@ -746,18 +746,54 @@ __global__ __launch_bounds__(512) void skinny_gemm_kernel(const GemmParams p) {
   }
 }
 
+// Tuning knobs for sweeps, read from the environment ONCE per process (the first GEMM call or
+// workspace query): what a query returned stays valid for every later call.
+//   TLF_GEMM_PLAN="bn,bm,splits,stages,occ[,kgroups,wn]"  forces one tiled plan
+//   TLF_GEMM_SKINNY_MAX_M   hand-over point between the skinny and the tiled kernel (0 ... 64)
+//   TLF_GEMM_SKINNY_TN      16-channel tiles per skinny workgroup (1, 2 or 4)
+//   TLF_GEMM_GROUP_N        N-tile columns per XCD patch
+struct GemmTuning {
+  bool has_plan = false;
+  int plan[7] = {0, 0, 0, 0, 0, 1, 0};
+  int skinny_max_m = kSkinnyMaxM;
+  int skinny_tn = 0;
+  int group_n = 0;
+};
+
+inline const GemmTuning &gemm_tuning() {
+  static const GemmTuning t = [] {
+    GemmTuning g;
+    if (const char *e = getenv("TLF_GEMM_PLAN")) {
+      int v[7] = {0, 0, 0, 0, 0, 1, 0};
+      if (sscanf(e, "%d,%d,%d,%d,%d,%d,%d", &v[0], &v[1], &v[2], &v[3], &v[4], &v[5], &v[6]) >= 5) {
+        g.has_plan = true;
+        for (int i = 0; i < 7; ++i) g.plan[i] = v[i];
+      }
+    }
+    if (const char *e = getenv("TLF_GEMM_SKINNY_MAX_M")) {
+      const int v = atoi(e);  // the skinny kernel covers at most 4 x 16 tokens
+      g.skinny_max_m = v < 0 ? 0 : v > 64 ? 64 : v;
+    }
+    if (const char *e = getenv("TLF_GEMM_SKINNY_TN")) {
+      const int v = atoi(e);
+      if (v == 1 || v == 2 || v == 4) g.skinny_tn = v;
+    }
+    if (const char *e = getenv("TLF_GEMM_GROUP_N")) g.group_n = atoi(e) > 0 ? atoi(e) : 1;
+    return g;
+  }();
+  return t;
+}
+
 template <bool W8>
 int launch_skinny(const GemmParams &p, hipStream_t stream) {
+  if (p.M > 64) return TLF_E_UNSUPPORTED;  // four 16-token MFMA tiles at most
   const int mt = (p.M + 15) / 16;
   const int tiles16 = (p.N + 15) / 16;
   // more channels per workgroup reuse the activation fragments, as long as the grid stays large
   int tn = 1;
   if (tiles16 >= 4 * 512) tn = 4;
   else if (tiles16 >= 2 * 512) tn = 2;
-  if (const char *e = getenv("TLF_GEMM_SKINNY_TN")) {  // tuning override
-    const int v = atoi(e);
-    if (v == 1 || v == 2 || v == 4) tn = v;
-  }
+  if (gemm_tuning().skinny_tn) tn = gemm_tuning().skinny_tn;
   const dim3 grid((tiles16 + tn - 1) / tn);
 #define TLF_SK(MT_, TN_) \
   hipLaunchKernelGGL((skinny_gemm_kernel<MT_, TN_, W8>), grid, dim3(512), 0, stream, p)
@@ -872,33 +908,24 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
   return g;
 }
 
-// TLF_GEMM_PLAN="bn,bm,splits,stages,occ" forces one plan (tuning sweeps); TLF_GEMM_SKINNY_MAX_M
-// moves the hand-over point between the skinny and the tiled kernel.
+// A forced plan (GemmTuning) replaces the planner's choice.
 inline bool plan_override(GemmPlan &g, int K) {
-  const char *e = getenv("TLF_GEMM_PLAN");
-  if (!e) return false;
-  int bn = 0, bm = 0, sp = 0, st = 0, occ = 0, kgr = 1, wn = 0;
-  if (sscanf(e, "%d,%d,%d,%d,%d,%d,%d", &bn, &bm, &sp, &st, &occ, &kgr, &wn) < 5) return false;
-  g.kgroups = kgr;
-  g.wn = wn;
+  const GemmTuning &t = gemm_tuning();
+  if (!t.has_plan) return false;
+  int sp = t.plan[2];
+  g.kgroups = t.plan[5];
+  g.wn = t.plan[6];
   const int ktiles = K / kBK;
   if (sp < 1) sp = 1;
   if (sp > ktiles) sp = ktiles;
   const int kt_per = (ktiles + sp - 1) / sp;
-  g.bn = bn; g.bm = bm; g.stages = st; g.occ = occ;
+  g.bn = t.plan[0]; g.bm = t.plan[1]; g.stages = t.plan[3]; g.occ = t.plan[4];
   g.k_per_split = kt_per * kBK;
   g.splits = (ktiles + kt_per - 1) / kt_per;
   return true;
 }
 
-inline int skinny_max_m() {
-  static int v = -1;
-  if (v < 0) {
-    v = kSkinnyMaxM;
-    if (const char *e = getenv("TLF_GEMM_SKINNY_MAX_M")) v = atoi(e);
-  }
-  return v;
-}
+inline int skinny_max_m() { return gemm_tuning().skinny_max_m; }
 
 // plan_out != nullptr: nothing is launched; the eight plan fields are written there instead and the
 // return code says whether a kernel instance exists for the plan.
@@ -965,7 +992,7 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   {
     const int cols = (p.n_tiles + 7) / 8;
     if (p.m_tiles >= 8) g.group_n = cols % 4 == 0 ? 4 : cols % 3 == 0 ? 3 : cols % 2 == 0 ? 2 : 1;
-    if (const char *e = getenv("TLF_GEMM_GROUP_N")) g.group_n = atoi(e) > 0 ? atoi(e) : 1;
+    if (gemm_tuning().group_n) g.group_n = gemm_tuning().group_n;
   }
   p.group_n = g.group_n;
   const int cols_per_xcd = ((p.n_tiles + 7) / 8 + g.group_n - 1) / g.group_n * g.group_n;
@@ -1077,7 +1104,7 @@ extern "C" size_t tlf_w8a16_gemm_workspace_bytes(int32_t M, int32_t N, int32_t K
   // fp32 partial sums of the plan's split of K (the larger of the int8 and the bf16 plan: both
   // entry points share this query); a tuning override may pick any split up to 16
   int splits = 16;
-  if (!getenv("TLF_GEMM_PLAN")) {
+  if (!gemm_tuning().has_plan) {
     int32_t p8[8], p16[8];
     if (launch_gemm<true>(nullptr, K, nullptr, nullptr, nullptr, M, N, K, nullptr, 0, nullptr, p8) == TLF_OK &&
         launch_gemm<false>(nullptr, K, nullptr, nullptr, nullptr, M, N, K, nullptr, 0, nullptr, p16) == TLF_OK)

@@ -44,6 +44,9 @@ class LLMEngine:
             if self.tokenizer is None:
                 raise ValueError("string prompts need a tokenizer; pass token-id lists instead")
             prompt = self.tokenizer.encode(prompt)
+        if len(prompt) > self.config.hf_config.max_position_embeddings:
+            raise ValueError(f"prompt of {len(prompt)} tokens exceeds max_position_embeddings "
+                             f"({self.config.hf_config.max_position_embeddings}): no RoPE row for its tail")
         self.scheduler.add(Sequence(prompt, sampling_params))
 
     def step(self):

@@ -57,6 +57,7 @@ class ModelRunner:
         self.fused_greedy = True      # all-greedy batches: LM head and argmax in one call
         self.graphs = {}
         self.graph_bs = []
+        self._stage = None            # pinned staging buffer of the eager steps' integer inputs (grow-only)
         with torch.inference_mode():
             self.warmup_model()
             self.allocate_kv_cache()
@@ -64,9 +65,19 @@ class ModelRunner:
                 self.capture_graphs()
 
     def exit(self):
-        self.graphs.clear()
-        self.graph_vars = None
+        """Release the graphs, the KV pool and the weights (whoever still holds this object holds no memory)."""
         torch.cuda.synchronize()
+        self.graphs.clear()
+        self.graph_vars = self.graph_host = self.graph_pack_dev = self.graph_pack_host = None
+        if getattr(self, "model", None) is not None:
+            for module in self.model.modules():
+                if hasattr(module, "k_cache") and hasattr(module, "v_cache"):
+                    module.k_cache = module.v_cache = torch.tensor([])
+        self.kv_cache = None
+        self.model = None
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
 
     def call(self, method_name, *args):
         return getattr(self, method_name)(*args)
@@ -107,10 +118,21 @@ class ModelRunner:
                 module.k_cache = self.kv_cache[0, layer_id]
                 module.v_cache = self.kv_cache[1, layer_id]
                 if self.kv_dtype != torch.bfloat16:
-                    # build-defined static per-head scales for the e4m3 cache
-                    module.k_scale = torch.full((hf.num_key_value_heads,), 1.0 / 16, dtype=torch.float32, device=self.device)
-                    module.v_scale = torch.full((hf.num_key_value_heads,), 1.0 / 16, dtype=torch.float32, device=self.device)
+                    # build-defined static per-head scales of the e4m3 cache (Config.kv_k_scale / kv_v_scale):
+                    # |x| above 448 * scale saturates
+                    module.k_scale = self._kv_scale(cfg.kv_k_scale, layer_id)
+                    module.v_scale = self._kv_scale(cfg.kv_v_scale, layer_id)
                 layer_id += 1
+
+    def _kv_scale(self, spec, layer_id: int) -> torch.Tensor:
+        """fp32 ``[Hkv]`` from a float (every head), ``[Hkv]`` values (every layer) or ``[L][Hkv]`` values."""
+        hkv = self.config.hf_config.num_key_value_heads
+        t = torch.as_tensor(spec, dtype=torch.float32)
+        if t.dim() == 2:
+            t = t[layer_id]
+        t = t.expand(hkv).contiguous() if t.dim() == 0 else t.contiguous()
+        assert t.shape == (hkv,) and bool((t > 0).all()), "KV scales: a positive float, [Hkv] or [L][Hkv]"
+        return t.to(self.device)
 
     # ------------------------------------------------------------------ per-step inputs
     def _upload(self, arrays: dict) -> dict:
@@ -121,11 +143,20 @@ class ModelRunner:
             total = (total + 15) // 16 * 16
             offs[k] = total
             total += arrays[k].nbytes
-        stage = torch.empty(max(total, 16), dtype=torch.uint8, pin_memory=True)
+        total = max(total, 16)
+        if self._stage is not None:
+            # the copy out of the buffer must be over before it is rewritten (normally it is: every
+            # step ends in the device -> host copy of its token ids)
+            self._stage_copied.synchronize()
+        if self._stage is None or self._stage.numel() < total:
+            self._stage = torch.empty(max(total, 1 << 20), dtype=torch.uint8, pin_memory=True)
+            self._stage_copied = torch.cuda.Event()
+        stage = self._stage[:total]
         sv = stage.numpy()
         for k in names:
             sv[offs[k]:offs[k] + arrays[k].nbytes] = arrays[k].reshape(-1).view(np.uint8)
         dev = stage.to(self.device, non_blocking=True)
+        self._stage_copied.record()
         out = dict(arrays)
         for k in names:
             a = arrays[k]
@@ -136,32 +167,43 @@ class ModelRunner:
     def prepare_block_tables(self, seqs):
         return torch.from_numpy(I.block_tables_array(seqs)).to(self.device)
 
+    def _temperatures_of(self, seqs) -> np.ndarray | None:
+        """fp32 temperatures of the step, or None for an all-greedy batch (the greedy kernel reads none)."""
+        t = np.asarray([s.temperature for s in seqs], dtype=np.float32)
+        self._all_greedy = bool((t == 0).all())
+        return None if self._all_greedy else t
+
     def prepare_prefill(self, seqs):
-        d = self._upload(I.prefill_inputs(seqs, self.block_size))
+        arrays = I.prefill_inputs(seqs, self.block_size)
+        arrays["temperatures"] = self._temperatures_of(seqs)       # rides in the step's one staging copy
+        d = self._upload(arrays)
+        self._temperatures = d["temperatures"]
         set_context(True, d["cu_seqlens_q"], d["cu_seqlens_k"], d["max_seqlen_q"], d["max_seqlen_k"],
                     d["slot_mapping"], None, d["block_tables"])
         return d["input_ids"], d["positions"]
 
     def prepare_decode(self, seqs):
-        d = self._upload(I.decode_inputs(seqs, self.block_size, self.config.decode_position_quirk))
+        arrays = I.decode_inputs(seqs, self.block_size, self.config.decode_position_quirk)
+        arrays["temperatures"] = self._temperatures_of(seqs)
+        d = self._upload(arrays)
+        self._temperatures = d["temperatures"]
         set_context(False, slot_mapping=d["slot_mapping"], context_lens=d["context_lens"], block_tables=d["block_tables"])
         return d["input_ids"], d["positions"]
 
     def prepare_sample(self, seqs):
-        t = np.asarray([s.temperature for s in seqs], dtype=np.float32)
-        self._all_greedy = bool((t == 0).all())
-        if self._all_greedy:
-            return None                      # the greedy kernel does not read temperatures
-        return torch.from_numpy(t).to(self.device, non_blocking=True)
+        """Temperatures of the step on the device (model_runner.py:230-236), None when all are 0: what the
+        step's ``prepare_prefill`` / ``prepare_decode`` / graph upload already carried over."""
+        return self._temperatures
 
     # ------------------------------------------------------------------ forward
     @torch.inference_mode()
     def run_hidden(self, input_ids, positions, is_prefill):
         """Final hidden states of the step's tokens (eager, or a graph replay with device-side inputs)."""
         bs = input_ids.size(0)
-        if is_prefill or self.enforce_eager or not self.graph_bs or bs > self.graph_bs[-1]:
-            return self.model(input_ids, positions)
         ctx = get_context()
+        if (is_prefill or self.enforce_eager or not self.graph_bs or bs > self.graph_bs[-1]
+                or ctx.block_tables is None or ctx.block_tables.size(1) > self.graph_max_blocks):
+            return self.model(input_ids, positions)      # a table wider than the graphs' static one runs eagerly
         gbs = next(x for x in self.graph_bs if x >= bs)
         gv = self.graph_vars
         if gbs != bs:      # padding rows: slot -1 (no cache write), length 0 (no cache read)
@@ -203,6 +245,11 @@ class ModelRunner:
             h["positions"][bs:gbs] = 0
             h["slot_mapping"][bs:gbs] = -1
             h["context_lens"][bs:gbs] = 0
+        t = self._temperatures_of(seqs)
+        self._temperatures = None
+        if t is not None:
+            h["temperatures"][:bs] = t
+            self._temperatures = self.graph_vars["temperatures"][:bs]
         self.graph_pack_dev.copy_(self.graph_pack_host, non_blocking=True)
         set_context(False)
         self.graphs[gbs].replay()
@@ -222,8 +269,8 @@ class ModelRunner:
                      and len(seqs) <= self.graph_bs[-1]
                      and max(len(s.block_table) for s in seqs) <= self.graph_max_blocks)
         if use_graph:
-            temperatures = self.prepare_sample(seqs)
-            token_ids = self.sample(self.run_decode_graph(seqs), temperatures)
+            hidden = self.run_decode_graph(seqs)
+            token_ids = self.sample(hidden, self.prepare_sample(seqs))
             reset_context()
             return token_ids
         input_ids, positions = self.prepare_prefill(seqs) if is_prefill else self.prepare_decode(seqs)
@@ -249,6 +296,7 @@ class ModelRunner:
         layout, off = {}, 0
         for name, dt, shape in (("input_ids", torch.int64, (max_bs,)), ("positions", torch.int64, (max_bs,)),
                                 ("slot_mapping", torch.int32, (max_bs,)), ("context_lens", torch.int32, (max_bs,)),
+                                ("temperatures", torch.float32, (max_bs,)),
                                 ("block_tables", torch.int32, (max_bs, max_blocks))):
             nbytes = int(np.prod(shape)) * torch.empty(0, dtype=dt).element_size()
             layout[name] = (off, nbytes, dt, shape)
@@ -256,7 +304,7 @@ class ModelRunner:
         self.graph_pack_dev = torch.zeros(off, dtype=torch.uint8, device=dev)
         self.graph_pack_host = torch.zeros(off, dtype=torch.uint8, pin_memory=True)
         host_np = self.graph_pack_host.numpy()
-        np_dt = {torch.int64: np.int64, torch.int32: np.int32}
+        np_dt = {torch.int64: np.int64, torch.int32: np.int32, torch.float32: np.float32}
         gv, self.graph_host = {}, {}
         for name, (o, nbytes, dt, shape) in layout.items():
             gv[name] = self.graph_pack_dev[o:o + nbytes].view(dt).view(*shape)

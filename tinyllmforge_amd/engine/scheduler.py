@@ -14,6 +14,10 @@ class Scheduler:
         self.max_num_seqs = config.max_num_seqs
         self.max_num_batched_tokens = config.max_num_batched_tokens
         self.eos = config.eos
+        # The RoPE table has max_position_embeddings rows and a decode step feeds position len(seq)
+        # (len(seq) - 1 without the reference's quirk): a sequence that would step past the table
+        # is finished instead (the reference indexes out of range there).
+        self.max_len = config.hf_config.max_position_embeddings + (0 if config.decode_position_quirk else 1)
         self.block_manager = BlockManager(config.num_kvcache_blocks, config.kvcache_block_size)
         self.waiting: deque[Sequence] = deque()
         self.running: deque[Sequence] = deque()
@@ -75,7 +79,7 @@ class Scheduler:
         for seq, tok in zip(seqs, token_ids):
             seq.append_token(tok)
             hit_eos = (not seq.ignore_eos) and tok == self.eos
-            if hit_eos or seq.num_completion_tokens == seq.max_tokens:
+            if hit_eos or seq.num_completion_tokens == seq.max_tokens or len(seq) >= self.max_len:
                 seq.status = SequenceStatus.FINISHED
                 self.block_manager.deallocate(seq)
                 self.running.remove(seq)

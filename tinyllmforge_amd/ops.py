@@ -30,16 +30,15 @@ _workspaces: dict = {}
 _retired: list = []   # outgrown buffers stay alive: a captured graph may still point at them
 
 
-def _workspace(nbytes: int, device, tag: str, zero: bool = False) -> torch.Tensor:
+def _workspace(nbytes: int, device, tag: str) -> torch.Tensor:
     """Grow-only scratch buffer per (device, tag).  Never freed, so pointers recorded in a
-    captured graph stay valid; ``zero`` buffers start zero-filled (decode arrival counters)."""
+    captured graph stay valid.  No kernel needs it cleared."""
     key = (device, tag)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         if ws is not None:
             _retired.append(ws)
-        alloc = torch.zeros if zero else torch.empty
-        ws = alloc(max(nbytes, 256), dtype=torch.uint8, device=device)
+        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
 

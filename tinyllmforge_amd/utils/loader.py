@@ -36,6 +36,11 @@ def load_tensor(model: nn.Module, packed: dict, name: str, tensor: torch.Tensor)
                 break
         model.get_submodule(module_name).load_quantized_shard(kind, tensor, shard_id)
         return
+    stem = name.rsplit(".", 2)[-2] if name.count(".") >= 1 else name
+    if stem in {target for target, _ in packed.values()}:
+        # already packed (``qkv_proj``, ``gate_up_proj``: a state dict taken from this model): whole copy
+        default_weight_loader(model.get_parameter(name), tensor)
+        return
     for key, (target, shard_id) in packed.items():
         if key in name:
             param = model.get_parameter(name.replace(key, target))
