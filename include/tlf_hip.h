@@ -38,6 +38,7 @@ extern "C" {
 #define TLF_E_ALIGN (-3)       /* a pointer or stride breaks the stated alignment    */
 #define TLF_E_WORKSPACE (-4)   /* workspace missing or too small                     */
 #define TLF_E_UNSUPPORTED (-5) /* a combination this build has no kernel for          */
+#define TLF_E_TOO_LARGE (-6)   /* a size beyond the fixed scratch of a no-allocation entry point */
 
 /* KV-cache element types */
 #define TLF_KV_BF16 0
@@ -166,6 +167,20 @@ size_t tlf_argmax_workspace_bytes(int32_t rows, int32_t vocab);
 int tlf_argmax(const void *logits, int64_t row_stride, int64_t *out,
                int32_t rows, int32_t vocab, void *workspace, size_t workspace_bytes,
                void *stream);
+
+/* tlf_argmax without a workspace argument and without any allocation.  No counterpart in the
+ * reference: it is for callers that cannot allocate device memory - code under hipGraph capture, tight
+ * serving loops, harnesses that forbid hipMalloc - and so cannot provide (or grow) the workspace that
+ * tlf_argmax asks for.  Same kernels and result as tlf_argmax; the partial keys live in a 1 MiB
+ * file-scope device array of the library (one copy per GPU, held until the process ends), which
+ * bounds rows <= tlf_argmax_noalloc_max_rows() (1024): more rows return TLF_E_TOO_LARGE.  The
+ * array's device address is looked up on the first call on each device (a host-side query, no
+ * allocation; make that first call outside a stream capture).  Calls on one GPU share the array:
+ * calls that may overlap in time (different streams) race; calls on one stream are ordered.
+ * Nothing needs clearing between calls (every key read was written by the same call). */
+int tlf_argmax_noalloc_max_rows(void);
+int tlf_argmax_noalloc(const void *logits, int64_t row_stride, int64_t *out,
+                       int32_t rows, int32_t vocab, void *stream);
 
 /* Sampler.forward with temperatures   replaces layers/sampler.py:13-21
  *

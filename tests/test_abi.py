@@ -63,6 +63,12 @@ def test_argument_rejection_happens_before_any_launch():
     assert lib.tlf_sample(a, 1024, None, a, 4, 1024, 0, 0, a, 1 << 20, None) == -1
     assert lib.tlf_sample(a, 1000, a, a, 4, 1024, 0, 0, a, 1 << 20, None) == -2
     assert lib.tlf_sample(a, 1024, a, a, 4, 1024, 0, 0, a, 8, None) == -4
+    # the entry point without allocation: its limit is enforced on the host, before anything touches a GPU
+    assert lib.tlf_argmax_noalloc_max_rows() == 1024
+    assert lib.tlf_argmax_noalloc(a, 64, a, 1025, 64, None) == -6 and b"scratch" in lib.tlf_error_string(-6)
+    assert lib.tlf_argmax_noalloc(None, 64, a, 4, 64, None) == -1
+    assert lib.tlf_argmax_noalloc(a, 60, a, 4, 64, None) == -2
+    assert lib.tlf_argmax_noalloc(a, 64, a, 0, 64, None) == 0
     m, n, k = 200, 4096, 12288
     assert lib.tlf_gemm_add_rmsnorm_workspace_bytes(m, n, k) >= lib.tlf_w8a16_gemm_workspace_bytes(m, n, k) + m * n * 2
     assert lib.tlf_gemm_argmax_workspace_bytes(256, 151936, 4096) >= 256 * (151936 // 32) * 8

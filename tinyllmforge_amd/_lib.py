@@ -34,6 +34,8 @@ SIGNATURES = {
     "tlf_silu_and_mul": (c_int32, [_P, _P, _I32, _I32, _P]),
     "tlf_argmax_workspace_bytes": (_SZ, [_I32, _I32]),
     "tlf_argmax": (c_int32, [_P, _I64, _P, _I32, _I32, _P, _SZ, _P]),
+    "tlf_argmax_noalloc_max_rows": (c_int32, []),
+    "tlf_argmax_noalloc": (c_int32, [_P, _I64, _P, _I32, _I32, _P]),
     "tlf_sample": (c_int32, [_P, _I64, _P, _P, _I32, _I32, c_uint64, c_uint64, _P, _SZ, _P]),
     "tlf_w8a16_gemm_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
     "tlf_w8a16_gemm": (c_int32, [_P, _I64, _P, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),

@@ -1,6 +1,8 @@
 // Single-pass, 128-bit vectorised elementwise / row-reduction kernels:
 // RMSNorm (+ residual), RoPE, SiLU-and-mul, embedding gather, greedy argmax.
 // All are HBM bound; each element is read once and written once.
+#include <mutex>
+
 #include "common.h"
 
 namespace tlf {
@@ -557,6 +559,59 @@ extern "C" int tlf_argmax(const void *logits, int64_t row_stride, int64_t *out, 
     return TLF_E_WORKSPACE;
   const int nchunks = argmax_chunks(rows, vocab);
   auto part = static_cast<unsigned long long *>(workspace);
+  hipLaunchKernelGGL(argmax_partial_kernel, dim3(nchunks, rows), dim3(256), 0,
+                     static_cast<hipStream_t>(stream),
+                     static_cast<const unsigned short *>(logits), row_stride, vocab, part, nchunks);
+  hipLaunchKernelGGL(argmax_final_kernel<64>, dim3(rows), dim3(64), 0,
+                     static_cast<hipStream_t>(stream), part, nchunks, out);
+  return launch_status();
+}
+
+// ---------------------------------------------------------------------------
+// Greedy argmax for callers that cannot allocate (code under hipGraph capture, tight serving loops,
+// harnesses that forbid hipMalloc): same two kernels as tlf_argmax, the partial keys go to a
+// file-scope device array instead of a caller workspace.  Each GPU the library runs on holds its own
+// copy of the array (1 MiB) until the process ends.
+constexpr int kNoAllocMaxRows = 1024;
+constexpr int kNoAllocMaxDevices = 64;
+static __device__ __align__(256) unsigned long long scratch[kNoAllocMaxRows * kArgmaxMaxChunks];
+
+// Device address of `scratch` on the current device, resolved once per device.  In host code the
+// array's name is only a handle for this lookup, never an address a kernel may be given.
+static int scratch_of_current_device(unsigned long long **out) {
+  static std::mutex mu;
+  static unsigned long long *ptrs[kNoAllocMaxDevices] = {};
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return static_cast<int>(e);
+  if (dev < 0 || dev >= kNoAllocMaxDevices) return TLF_E_UNSUPPORTED;
+  std::lock_guard<std::mutex> lock(mu);
+  if (ptrs[dev] == nullptr) {
+    void *p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (p == nullptr) return static_cast<int>(hipErrorInvalidSymbol);
+    ptrs[dev] = static_cast<unsigned long long *>(p);
+  }
+  *out = ptrs[dev];
+  return TLF_OK;
+}
+
+extern "C" int tlf_argmax_noalloc_max_rows(void) { return kNoAllocMaxRows; }
+
+extern "C" int tlf_argmax_noalloc(const void *logits, int64_t row_stride, int64_t *out, int32_t rows,
+                                  int32_t vocab, void *stream) {
+  if (rows == 0) return TLF_OK;
+  if (!logits || !out) return TLF_E_NULL;
+  if (rows < 0 || vocab <= 0 || row_stride < vocab) return TLF_E_SHAPE;
+  if (rows > kNoAllocMaxRows) return TLF_E_TOO_LARGE;
+  if (!aligned16(logits) || row_stride % 8) return TLF_E_ALIGN;
+  unsigned long long *part = nullptr;
+  const int rc = scratch_of_current_device(&part);
+  if (rc != TLF_OK) return rc;
+  // every (row, chunk) key that the second kernel reads is written by the first one in this call:
+  // nothing of an earlier call's contents is read, so the array needs no clearing
+  const int nchunks = argmax_chunks(rows, vocab);
   hipLaunchKernelGGL(argmax_partial_kernel, dim3(nchunks, rows), dim3(256), 0,
                      static_cast<hipStream_t>(stream),
                      static_cast<const unsigned short *>(logits), row_stride, vocab, part, nchunks);

@@ -11,6 +11,7 @@ extern "C" const char *tlf_error_string(int code) {
     case TLF_E_ALIGN: return "a pointer or stride is not 16-byte aligned";
     case TLF_E_WORKSPACE: return "workspace missing, misaligned or too small";
     case TLF_E_UNSUPPORTED: return "no kernel for this combination";
+    case TLF_E_TOO_LARGE: return "size beyond the fixed scratch array of this no-allocation entry point";
     default: break;
   }
   if (code > 0) return hipGetErrorString(static_cast<hipError_t>(code));
