@@ -231,7 +231,7 @@ def bench_gemm(args, ms=(1, 16, 64, 128, 256, 2048, 8192)):
     rows = []
     for name, (N, K) in GEMM_SHAPES.items():
         copies = max(2, -(-(768 << 20) // (N * K)))
-        wqs = [torch.randint(-127, 128, (N, K), device="cuda", dtype=torch.int8) for _ in range(copies)]
+        wqs = [P.pack_w8(torch.randint(-127, 128, (N, K), device="cuda", dtype=torch.int8)) for _ in range(copies)]
         scale = torch.rand(N, device="cuda") * 9e-3 + 1e-3
         for M in ms:
             x = torch.randn(M, K, device="cuda").to(torch.bfloat16)

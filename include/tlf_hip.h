@@ -205,12 +205,18 @@ int tlf_sample(const void *logits, int64_t row_stride, const float *temperatures
  *
  *   y[m, n] = bf16( (sum_k x[m, k] * float(wq[n, k])) * scale[n] )   fp32 accumulate
  *
- * x: bf16 [M, K] row stride x_stride (elements); wq: int8 [N, K] contiguous;
- * scale: fp32 [N]; y: bf16 [M, N] contiguous.  K % 64 == 0, N % 16 == 0.
+ * x: bf16 [M, K] row stride x_stride (elements); wq: the int8 weight IN TILE ORDER, i.e. the output
+ * of tlf_w8a16_pack_weight for the row-major [N, K] weight (same bytes, re-ordered so that every wave
+ * reads contiguous runs: the 16-byte piece W[n, 16 a .. 16 a + 15] sits at byte
+ * ((n / 32) * (K / 32) + a / 2) * 1024 + (a % 2) * 512 + (n % 32) * 16; rows are padded to a multiple of
+ * 32); scale: fp32 [N]; y: bf16 [M, N] contiguous.  K % 64 == 0, N % 16 == 0.  Every W8A16 entry point
+ * below takes the weight in this order.
  * workspace: fp32 partial sums when the kernel plan for (M, N, K) splits K across workgroups
  * (few output tiles, long K); tlf_w8a16_gemm_workspace_bytes gives the size for this and for
  * tlf_bf16_gemm (0 when neither plan splits), 16-byte aligned.
  */
+size_t tlf_w8a16_packed_bytes(int32_t N, int32_t K);   /* = round_up(N, 32) * K */
+int tlf_w8a16_pack_weight(const void *wq_rowmajor, void *packed, int32_t N, int32_t K, void *stream);
 size_t tlf_w8a16_gemm_workspace_bytes(int32_t M, int32_t N, int32_t K);
 int tlf_w8a16_gemm(const void *x, int64_t x_stride, const void *wq, const float *scale,
                    void *y, int32_t M, int32_t N, int32_t K,
@@ -234,7 +240,7 @@ int tlf_bf16_gemm(const void *x, int64_t x_stride, const void *w, void *y,
  *   g = bf16(scale[..] * sum_k x[m,k] wq[.., k]),  u likewise
  *   y[m, c] = bf16( bf16(silu(g[m, c])) * u[m, c] )          y: bf16 [M, N/2] contiguous
  *
- * wq / scale rows are INTERLEAVED: rows 16 j .. 16 j + 7 are gate channels 8 j .. 8 j + 7 and rows
+ * wq / scale rows are INTERLEAVED (before tlf_w8a16_pack_weight): rows 16 j .. 16 j + 7 are gate channels 8 j .. 8 j + 7 and rows
  * 16 j + 8 .. 16 j + 15 the matching up channels (N = 2 x intermediate size, N % 16 == 0), so that
  * both halves of a product sit in one lane's accumulators.  Bit-identical to tlf_w8a16_gemm on
  * the same interleaved weight followed by tlf_silu_and_mul on the de-interleaved result.

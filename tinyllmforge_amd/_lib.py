@@ -37,6 +37,8 @@ SIGNATURES = {
     "tlf_argmax_noalloc_max_rows": (c_int32, []),
     "tlf_argmax_noalloc": (c_int32, [_P, _I64, _P, _I32, _I32, _P]),
     "tlf_sample": (c_int32, [_P, _I64, _P, _P, _I32, _I32, c_uint64, c_uint64, _P, _SZ, _P]),
+    "tlf_w8a16_packed_bytes": (_SZ, [_I32, _I32]),
+    "tlf_w8a16_pack_weight": (c_int32, [_P, _P, _I32, _I32, _P]),
     "tlf_w8a16_gemm_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
     "tlf_w8a16_gemm": (c_int32, [_P, _I64, _P, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),
     "tlf_bf16_gemm": (c_int32, [_P, _I64, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),

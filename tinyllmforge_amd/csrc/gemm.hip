@@ -9,15 +9,27 @@
 // the per-channel scale is a per-register constant and the bf16 result is
 // written as 8-byte pieces of a y row.
 //
-// Two kernels: a tiled one whose K-tiles travel global -> LDS without passing
-// through registers (gemm_dlds_kernel, more than 16 tokens) and a skinny one
-// that streams W straight into MFMA operand registers (skinny_gemm_kernel).
+// int8 weights are held in TILE ORDER (tlf_w8a16_pack_weight), not row-major: the 16-byte atom
+// W[n, 16 a .. 16 a + 15] of row n sits at byte
+//     ((n / 32) * (K / 32) + a / 2) * 1024 + (a % 2) * 512 + (n % 32) * 16,
+// i.e. 32 rows x 32 K values form one contiguous 1 KiB chunk whose 64 atoms are, in order, the
+// A operands of v_mfma_f32_32x32x16_bf16 for lanes 0..63 (lane = (a % 2) * 32 + n % 32), and the
+// chunks of one 32-row group follow each other along K.  A wave that owns a 32-row group streams
+// one contiguous run with 1 KiB per load instruction (measured on MI355X: 5.4 TB/s, against
+// 3.3 TB/s for the 32 rows x 32 bytes per instruction that row-major weights give this MFMA).
+// bf16 weights stay row-major (the reference's nn.Linear layout).
+//
+// Three kernels: a tiled one whose K-tiles travel global -> LDS without passing through
+// registers (gemm_dlds_kernel), a W-streaming one for decode-size batches in which every wave
+// streams its own weight rows global -> registers and only the activations go through LDS
+// (gemm_wstream_kernel), and a skinny one for a handful of tokens (skinny_gemm_kernel).
 //
 // Tile order is XCD aware: hardware deals workgroups round-robin to the 8 XCDs
 // (each with a private L2), so workgroup b belongs to XCD b % 8.  Each XCD is
 // given whole columns of N-tiles, so the workgroups that share an L2 share W
 // and x panels and step through K together.
 #include <stdio.h>
+#include <type_traits>
 #include <stdlib.h>
 
 #include "common.h"
@@ -200,7 +212,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
 #define TLF_DL_ISSUE_SETUP(XS, WS, T)                                                             \
   const int kt_ = min((T), nkt - 1);                                                              \
   const unsigned char *xg_ = xbase + static_cast<int64_t>(kt_) * (kBK * 2);                       \
-  const unsigned char *wg_ = wbase + static_cast<int64_t>(kt_) * kWRow;                           \
+  const unsigned char *wg_ = wbase + static_cast<int64_t>(kt_) * kWStep;                          \
   const unsigned int xl_ = TLF_DL_LDSADDR(XS) + set_u * kXBytes + wave_u * 1024,                  \
                      wl_ = TLF_DL_LDSADDR(WS) + set_u * kWBytes + wave_u * 1024;
 // Slice PART of 4 of the copies.  The copies are spread over the step, between the MFMA groups:
@@ -320,6 +332,7 @@ void gemm_dlds_kernel(const GemmParams p) {
   constexpr int WN = BN / WAVES_N, WM = BM / WAVES_M;
   constexpr int TN = WN / 32, TM = WM / 32;
   constexpr int kWRow = W8 ? kBK : kBK * 2;   // bytes of one W row in a K-tile
+  constexpr int kWStep = W8 ? 2 * 1024 : kBK * 2;  // global bytes from one K-tile to the next (int8: two 1 KiB chunks)
   constexpr int kPass = NW * 1024;            // bytes one copy instruction moves per wave set
   constexpr int XP = BM * 128 / kPass;        // copies per lane and stage: x
   constexpr int WP = BN * kWRow / kPass;      // ... and W
@@ -365,7 +378,9 @@ void gemm_dlds_kernel(const GemmParams p) {
   // copy side: byte offset of this lane's piece for each pass, relative to the tile's first row
   // (rows past the end are clamped to the last row; their results are never stored)
   const unsigned char *xbase = p.x + m0 * p.ldx_bytes + static_cast<int64_t>(k_begin) * 2;
-  const unsigned char *wbase = p.w + n0 * ldw_bytes + static_cast<int64_t>(k_begin) * (W8 ? 1 : 2);
+  // int8 weights are in tile order: the row term is part of woff, the K term counts 1 KiB chunks of 32
+  const unsigned char *wbase = W8 ? p.w + static_cast<int64_t>(k_begin / 32) * 1024
+                                  : p.w + n0 * ldw_bytes + static_cast<int64_t>(k_begin) * 2;
   unsigned int xoff[XP], woff[WP];
   {
     const int rl = wave * 8 + (lane >> 3);  // row inside a pass of NW * 8 rows
@@ -380,8 +395,9 @@ void gemm_dlds_kernel(const GemmParams p) {
       const int pw = (lane & 3) ^ ((rw >> 2) & 3);
 #pragma unroll
       for (int q = 0; q < WP; ++q) {
-        const int row = min(n0 + q * (NW * 16) + rw, p.N - 1) - n0;
-        woff[q] = static_cast<unsigned int>(row * ldw_bytes + pw * 16);
+        // atom (row n, piece pw of the K-tile) of the tile-ordered weight, relative to the K-tile's first chunk
+        const int n = min(n0 + q * (NW * 16) + rw, p.N - 1);
+        woff[q] = static_cast<unsigned int>((n >> 5) * (p.K * 32) + (pw >> 1) * 1024 + (pw & 1) * 512 + (n & 31) * 16);
       }
     } else {
 #pragma unroll
@@ -477,6 +493,215 @@ void gemm_dlds_kernel(const GemmParams p) {
     }
   }
   gemm_epilogue<TN, TM, WN, WM, W8>(p, acc, m0, n0, wn, wm, r, kg, split);
+}
+
+// ---------------------------------------------------------------------------
+// W-streaming kernel for decode-size batches, int8 weights in tile order.
+//
+// At these sizes every weight byte is used once per token tile and the kernel lives or dies by how
+// the 256 CUs pull the weight matrix out of HBM.  A workgroup owns 128 channels and all tokens.
+// Its 4 x KG compute waves are 4 side by side along N times KG along K: wave (n, kh) owns one
+// 32-row group of W for the kh-th part of the workgroup's K range and streams it global -> registers:
+// one contiguous run, 1 KiB per load instruction, PF K-tiles (2 KiB each) in flight per wave, no LDS
+// and no workgroup barrier on the weight side; each lane's 16 bytes are its MFMA A operand after the
+// int8 -> bf16 conversion.  Only the activations are shared: one more wave does nothing but copy
+// x K-tiles (all tokens x 64 K values, one per K part) global -> LDS into a ring of NS stages, with a
+// load counter of its own, so the compute waves' counted waits see nothing but their weight loads;
+// one barrier per step hands a stage over.  KG = 2 puts two compute waves on every SIMD, which take
+// turns in the matrix pipe while the other one waits for LDS or converts; their accumulators are
+// added through LDS at the end.  Accumulator layout and epilogue are those of the tiled kernel.
+constexpr int kWsCols = 4;  // compute waves side by side along N (128 channels per workgroup)
+
+template <int TM, int NS, int PF, int KG>
+__global__ __launch_bounds__((kWsCols * KG + 1) * 64) __attribute__((amdgpu_waves_per_eu(1, KG + 1)))
+void gemm_wstream_kernel(const GemmParams p) {
+  constexpr int BM = TM * 32;
+  constexpr int kCompute = kWsCols * KG;
+  constexpr int kXBytes = BM * 128;        // one x tile: BM rows of 64 bf16
+  constexpr int kStage = KG * kXBytes;     // one stage: the x tile of every K part
+  constexpr int XP = BM / 8;               // copy instructions per x tile (8 rows of 128 bytes each)
+  constexpr int kReduce = (KG - 1) * kWsCols * TM * 16 * 64 * 4;
+  constexpr int kPool = NS * kStage > kReduce ? NS * kStage : kReduce;
+  static_assert(NS >= 2 && kPool <= 160 * 1024, "the stages must fit LDS");
+  static_assert((NS - 2) * KG * XP <= 63, "vmcnt range");
+  static_assert(PF == 2 || PF == 4 || PF == 8, "2, 4 or 8 tiles in flight");
+  __shared__ __attribute__((aligned(1024))) unsigned char pool[kPool];
+  const int lane = threadIdx.x & 63;
+  const unsigned int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int split = blockIdx.y;
+  const int k_begin = split * p.k_per_split;
+  const int nh = (min(p.K, k_begin + p.k_per_split) - k_begin) / kBK / KG;  // steps = K-tiles per K part, >= 1 (host)
+  const int n0 = blockIdx.x * (kWsCols * 32);
+
+  if (wave == kCompute) {
+    // ---- the copy wave: step s brings tile s of every K part to stage s % NS; piece c of LDS row R
+    // sits at c ^ ((R >> 1) & 7)
+    const unsigned char *xbase = p.x + static_cast<int64_t>(k_begin) * 2;
+    unsigned int xoff[XP];
+#pragma unroll
+    for (int q = 0; q < XP; ++q) {
+      const int R = q * 8 + (lane >> 3);
+      const int piece = (lane & 7) ^ ((R >> 1) & 7);
+      xoff[q] = static_cast<unsigned int>(min(R, p.M - 1) * p.ldx_bytes + piece * 16);  // rows past M: a copy of the last row
+    }
+    const unsigned int lds0 = TLF_DL_LDSADDR(pool);
+#define TLF_WS_ISSUE(S, STAGE)                                                             \
+  {                                                                                        \
+    const int s_ = min((S), nh - 1);                                                       \
+    _Pragma("unroll") for (int h = 0; h < KG; ++h) {                                       \
+      const unsigned char *xg_ = xbase + static_cast<int64_t>(h * nh + s_) * (kBK * 2);    \
+      const unsigned int xl_ = lds0 + static_cast<unsigned int>(STAGE) * kStage + h * kXBytes; \
+      _Pragma("unroll") for (int q = 0; q < XP; ++q) TLF_DL_COPY(xoff[q], xg_, xl_ + q * 1024); \
+    }                                                                                      \
+  }
+#pragma unroll
+    for (int s = 0; s < NS - 1; ++s) TLF_WS_ISSUE(s, s)
+    int stage = NS - 1;
+    for (int s = 0; s < nh; ++s) {
+      // step s has landed once at most the NS - 2 steps after it are in flight; the barrier publishes it
+      // and says that every compute wave is done with step s - 1, whose stage the next copy overwrites
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"((NS - 2) * KG * XP) : "memory");
+      TLF_WS_ISSUE(s + NS - 1, stage)
+      stage = stage + 1 == NS ? 0 : stage + 1;
+    }
+#undef TLF_WS_ISSUE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // no copy may land after the stages are re-used or released
+    if constexpr (KG > 1) {  // the two barriers of the accumulator exchange
+      asm volatile("s_barrier" ::: "memory");
+      asm volatile("s_barrier" ::: "memory");
+    }
+    return;
+  }
+
+  // ---- compute waves
+  const int r = lane & 31, kg = lane >> 5;
+  const int col = static_cast<int>(wave) % kWsCols, kh = static_cast<int>(wave) / kWsCols;
+  const int nt = n0 / 32 + col;
+  const bool has_rows = nt * 32 < p.N;
+  const int ntc = has_rows ? nt : (p.N - 1) / 32;  // a wave without rows streams the last group and stores nothing
+  // chunk c (32 K values of the 32-row group) of this wave's K part is the 1 KiB at wp + c * 1024
+  const unsigned char *wp = p.w + (static_cast<int64_t>(ntc) * (p.K / 32) + k_begin / 32 + kh * nh * 2) * 1024 + lane * 16;
+  const int xrow = kh * kXBytes + r * 128;
+  int xq[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)  // chunk c = i / 2, half h = i % 2 of the tile: x piece 4 c + 2 kg + h
+    xq[i] = (((i >> 1) * 4 + kg * 2 + (i & 1)) ^ ((r >> 1) & 7)) * 16;
+
+  floatx16 acc[1][TM];
+#pragma unroll
+  for (int j = 0; j < TM; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[0][j][v] = 0.f;
+
+  // Tile t of this wave's stream = chunks 2 t and 2 t + 1.  Every load below is unconditional (an index
+  // past the end re-reads the last tile, an L2 hit): with branches around them the compiler gives up
+  // counting and waits for ALL outstanding loads before every use, which is the end of the prefetch.
+  auto load_tile = [&](int t, u32x4 (&dst)[2]) {
+    const unsigned char *src = wp + static_cast<int64_t>(min(t, nh - 1)) * 2048;
+    dst[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src));
+    dst[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + 1024));
+  };
+  // quarter q of a tile's 32 weights per lane -> the A operand of MFMA group q
+  auto convert_quarter = [&](const u32x4 (&raw)[2], int q, bf16x8 &a) {
+    const unsigned int d0 = (q & 1) ? raw[q >> 1].z : raw[q >> 1].x;
+    const unsigned int d1 = (q & 1) ? raw[q >> 1].w : raw[q >> 1].y;
+    const uint2 c0 = cvt4_i8_bf16(d0), c1 = cvt4_i8_bf16(d1);
+    Pack16 t;
+    t.u = make_uint4(c0.x, c0.y, c1.x, c1.y);
+    a = t.v;
+  };
+  int cur = 0;
+  uint4 bfrag[2][TM];
+  auto read_group = [&](int g, uint4 (&dst)[TM]) {
+    const unsigned char *xs = pool + cur * kStage + xrow + xq[g];
+#pragma unroll
+    for (int j = 0; j < TM; ++j) dst[j] = *reinterpret_cast<const uint4 *>(xs + j * (32 * 128));
+  };
+  auto mfma_group = [&](const bf16x8 &a, const uint4 (&b)[TM]) {
+#pragma unroll
+    for (int j = 0; j < TM; ++j) {
+      Pack16 t;
+      t.u = b[j];
+      acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, t.v, acc[0][j], 0, 0, 0);
+    }
+  };
+
+  u32x4 wreg[PF][2];
+#pragma unroll
+  for (int u = 0; u < PF; ++u) load_tile(u, wreg[u]);
+  // One step: tile t = t0 + u of this wave's K part.  GUARDED = the last trip, where tiles may lie past
+  // the end of the stream; the trips before it run without a branch.  Within a step the x fragments of
+  // MFMA group g + 1 are requested before the MFMAs of group g are issued (two fragment buffers).
+  auto tile_step = [&](auto guarded, int t0, auto uc) {
+    constexpr bool G = decltype(guarded)::value;
+    constexpr int u = decltype(uc)::value;
+    const int t = t0 + u;
+    const bool live = !G || t < nh;  // uniform
+    bf16x8 a[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) convert_quarter(wreg[u], q, a[q]);
+    load_tile(t + PF, wreg[u]);  // the registers just read take tile t + PF
+    if (live) {
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");  // step t is in stage cur
+      read_group(0, bfrag[0]);
+      read_group(1, bfrag[1]);
+      mfma_group(a[0], bfrag[0]);
+      read_group(2, bfrag[0]);
+      mfma_group(a[1], bfrag[1]);
+      read_group(3, bfrag[1]);
+      mfma_group(a[2], bfrag[0]);
+      mfma_group(a[3], bfrag[1]);
+      cur = cur + 1 == NS ? 0 : cur + 1;
+    }
+  };
+  auto trip = [&](auto guarded, int t0) {
+    tile_step(guarded, t0, std::integral_constant<int, 0>{});
+    tile_step(guarded, t0, std::integral_constant<int, 1>{});
+    if constexpr (PF > 2) {
+      tile_step(guarded, t0, std::integral_constant<int, 2>{});
+      tile_step(guarded, t0, std::integral_constant<int, 3>{});
+    }
+    if constexpr (PF > 4) {
+      tile_step(guarded, t0, std::integral_constant<int, 4>{});
+      tile_step(guarded, t0, std::integral_constant<int, 5>{});
+      tile_step(guarded, t0, std::integral_constant<int, 6>{});
+      tile_step(guarded, t0, std::integral_constant<int, 7>{});
+    }
+  };
+  // full trips run unguarded; one guarded trip takes the rest (0 .. PF - 1 tiles)
+  const int full = nh / PF;
+  int t0 = 0;
+  for (int i = 0; i < full; ++i, t0 += PF) trip(std::false_type{}, t0);
+  if (t0 < nh) trip(std::true_type{}, t0);
+
+  if constexpr (KG > 1) {
+    // add the K parts' accumulators: parts 1.. park theirs in LDS (lane-major, conflict free), part 0 adds.
+    // The copy wave has drained its copies before it joins the first barrier.
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    float *red = reinterpret_cast<float *>(pool);
+    const int slot = col * 64 + lane;
+    if (kh > 0) {
+      float *dst = red + (kh - 1) * (kWsCols * TM * 16 * 64) + slot;
+#pragma unroll
+      for (int j = 0; j < TM; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dst[(j * 16 + v) * (kWsCols * 64)] = acc[0][j][v];
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    if (kh > 0) return;
+#pragma unroll
+    for (int g = 0; g < KG - 1; ++g) {
+      const float *src = red + g * (kWsCols * TM * 16 * 64) + slot;
+#pragma unroll
+      for (int j = 0; j < TM; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[0][j][v] += src[(j * 16 + v) * (kWsCols * 64)];
+    }
+  }
+  if (has_rows)
+    gemm_epilogue<1, TM, 32, BM, true>(p, acc, 0, n0, col, 0, r, kg, split);
 }
 #undef TLF_DL_STEP
 #undef TLF_DL_STEP2
@@ -621,7 +846,10 @@ __global__ __launch_bounds__(512) void skinny_gemm_kernel(const GemmParams p) {
   for (int t = 0; t < TN; ++t) {
     const int n = n0 + t * 16 + r;
     wok[t] = n < p.N;
-    wrow[t] = p.w + static_cast<int64_t>(wok[t] ? n : 0) * ldw;
+    const int nn = wok[t] ? n : 0;
+    // int8: tile-ordered weight, this lane's atoms are (row nn, 16 K values 64 kb + 16 g ..)
+    wrow[t] = W8 ? p.w + static_cast<int64_t>(nn >> 5) * p.K * 32 + (nn & 31) * 16 + (g >> 1) * 1024 + (g & 1) * 512
+                 : p.w + static_cast<int64_t>(nn) * ldw;
   }
   const unsigned char *xrow[MT];
   bool xok[MT];
@@ -642,7 +870,7 @@ __global__ __launch_bounds__(512) void skinny_gemm_kernel(const GemmParams p) {
       for (int t = 0; t < TN; ++t) {
         if (W8) {
           wraw[u][t][0] = make_uint4(0, 0, 0, 0);
-          if (kb < kb_end && wok[t]) wraw[u][t][0] = load_nt_u4(wrow[t] + kb * kBK + g * 16);
+          if (kb < kb_end && wok[t]) wraw[u][t][0] = load_nt_u4(wrow[t] + static_cast<int64_t>(kb) * 2048);
         } else {
           wraw[u][t][0] = make_uint4(0, 0, 0, 0);
           wraw[u][t][W8 ? 0 : 1] = make_uint4(0, 0, 0, 0);
@@ -752,12 +980,20 @@ __global__ __launch_bounds__(512) void skinny_gemm_kernel(const GemmParams p) {
 //   TLF_GEMM_SKINNY_MAX_M   hand-over point between the skinny and the tiled kernel (0 ... 64)
 //   TLF_GEMM_SKINNY_TN      16-channel tiles per skinny workgroup (1, 2 or 4)
 //   TLF_GEMM_GROUP_N        N-tile columns per XCD patch
+//   TLF_GEMM_WSTREAM_M="lo,hi"  token range served by the W-streaming kernel ("0,0": never)
+//   TLF_GEMM_WSTREAM_SPLITS     its split of K across workgroups
+//   TLF_GEMM_WSTREAM_KG         its K parts inside a workgroup (1 or 2)
+//   TLF_GEMM_WSTREAM_FORCE=1    take it for every shape in its token range, not only where it measured faster
 struct GemmTuning {
   bool has_plan = false;
   int plan[7] = {0, 0, 0, 0, 0, 1, 0};
   int skinny_max_m = kSkinnyMaxM;
   int skinny_tn = 0;
   int group_n = 0;
+  int ws_min_m = kSkinnyMaxM + 1, ws_max_m = 128;  // token range of the W-streaming kernel (int8 weights)
+  int ws_splits = 0;                               // forced split of K for it
+  int ws_kg = 0;                                   // forced K parts per workgroup (1 or 2)
+  bool ws_force = false;                           // take it for every shape in its token range
 };
 
 inline const GemmTuning &gemm_tuning() {
@@ -779,6 +1015,16 @@ inline const GemmTuning &gemm_tuning() {
       if (v == 1 || v == 2 || v == 4) g.skinny_tn = v;
     }
     if (const char *e = getenv("TLF_GEMM_GROUP_N")) g.group_n = atoi(e) > 0 ? atoi(e) : 1;
+    if (const char *e = getenv("TLF_GEMM_WSTREAM_M")) {
+      int lo = 0, hi = 0;
+      if (sscanf(e, "%d,%d", &lo, &hi) == 2) {
+        g.ws_min_m = lo < 1 ? 1 : lo;
+        g.ws_max_m = hi > 256 ? 256 : hi;
+      }
+    }
+    if (const char *e = getenv("TLF_GEMM_WSTREAM_SPLITS")) g.ws_splits = atoi(e) > 0 ? atoi(e) : 0;
+    if (const char *e = getenv("TLF_GEMM_WSTREAM_FORCE")) g.ws_force = atoi(e) != 0;
+    if (const char *e = getenv("TLF_GEMM_WSTREAM_KG")) g.ws_kg = atoi(e) == 1 || atoi(e) == 2 ? atoi(e) : 0;
     return g;
   }();
   return t;
@@ -821,7 +1067,49 @@ struct GemmPlan {
   int group_n = 1;    // N-tile columns per XCD patch
   int kgroups = 1;    // wave sets splitting K inside a workgroup
   int wn = 0;         // waves along the channel side of the tile (0: the tile's default layout)
+  bool wstream = false;  // the W-streaming kernel: bn = 128 channels, bm = all tokens rounded to 32
 };
+
+// Plan of the W-streaming kernel (int8 weights, at most 256 tokens).  A workgroup takes 128 channels
+// and all tokens; K is split across workgroups until about 256 of them exist (small N), each split
+// keeping at least 8 K-tiles.  The fused activation needs whole sums, so it takes the kernel only
+// when N alone fills the machine.
+inline bool plan_wstream(int M, int N, int K, int act, GemmPlan &g) {
+  const GemmTuning &t = gemm_tuning();
+  if (t.has_plan || M < t.ws_min_m || M > t.ws_max_m || M < 1 || act == 2) return false;
+  const int n_wg = (N + 127) / 128;
+  const int ktiles = K / kBK;
+  int splits = 1;
+  // Measured against the tiled plans on the Qwen3-8B projections with cold weights: a wide N (gate_up)
+  // wins at every size up to 128 tokens (24 / 28 / 37 us at 32 / 64 / 128 tokens against 36 / 38 / 43);
+  // a narrow N needs a split of K, whose activation traffic and partial sums grow with the token count:
+  // it wins up to 32 tokens (qkv 12 us against 15, o_proj 12 against 13.5) and, with a long K
+  // (down projection), up to 96 (17 / 22 / 25 us at 32 / 64 / 96 tokens against 26 / 27 / 28).
+  if (!t.ws_force && n_wg < 96 && !(M <= 32 || (ktiles >= 128 && M <= 96))) return false;
+  if (act) {
+    if (n_wg < 96) return false;
+  } else {
+    splits = (256 + n_wg / 2) / n_wg;
+    if (splits > ktiles / 8) splits = ktiles / 8;
+    if (splits > 16) splits = 16;
+    if (t.ws_splits) splits = t.ws_splits < ktiles ? t.ws_splits : ktiles;
+    if (splits < 1) splits = 1;
+  }
+  const int kt_per = (ktiles + splits - 1) / splits;
+  const int tm = (M + 31) / 32;
+  g.wstream = true;
+  g.bn = 128;
+  g.bm = tm * 32;
+  int kg = ktiles % 2 == 0 && kt_per >= 4 ? 2 : 1;
+  if (t.ws_kg && (t.ws_kg == 1 || ktiles % 2 == 0)) kg = t.ws_kg;
+  g.stages = kg == 2 && tm >= 3 ? 3 : 4;
+  g.occ = kg;
+  g.kgroups = kg;
+  g.group_n = 1;
+  g.k_per_split = kt_per * kBK;
+  g.splits = (ktiles + kt_per - 1) / kt_per;
+  return true;
+}
 
 // Tile, stage and split-K choice, from sweeps over the Qwen3-8B projection shapes on MI355X
 // (M from 24 to 8192, int8 and bf16 weights).  Few tiles: small tiles and a split of K so that
@@ -956,8 +1244,11 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
     if (act == 2) return TLF_E_UNSUPPORTED;  // the caller stages the logits and runs tlf_argmax
     return launch_skinny<W8>(p, stream);
   }
-  GemmPlan g = plan_gemm(M, N, K, W8);
-  plan_override(g, K);
+  GemmPlan g;
+  if (!(W8 && plan_wstream(M, N, K, act, g))) {
+    g = plan_gemm(M, N, K, W8);
+    plan_override(g, K);
+  }
   if (act) {  // the activation needs whole sums: no split of K across workgroups
     g.splits = 1;
     g.k_per_split = K;
@@ -998,6 +1289,21 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   const int cols_per_xcd = ((p.n_tiles + 7) / 8 + g.group_n - 1) / g.group_n * g.group_n;
   const dim3 grid(cols_per_xcd * 8 * p.m_tiles, g.splits);
   bool launched = false;
+  if constexpr (W8) {
+    if (g.wstream) {
+      const dim3 wgrid(p.n_tiles, g.splits);
+#define TLF_WS(TM_, NS_, PF_, KG_)                                                                  \
+  if (!launched && g.bm == TM_ * 32 && g.kgroups == KG_) {                                          \
+    if (!dry)                                                                                       \
+      hipLaunchKernelGGL((gemm_wstream_kernel<TM_, NS_, PF_, KG_>), wgrid,                          \
+                         dim3((kWsCols * KG_ + 1) * 64), 0, stream, p);                             \
+    launched = true;                                                                                \
+  }
+      TLF_WS(1, 4, 8, 1) TLF_WS(2, 4, 8, 1) TLF_WS(3, 4, 8, 1) TLF_WS(4, 4, 8, 1)
+      TLF_WS(1, 4, 4, 2) TLF_WS(2, 4, 4, 2) TLF_WS(3, 3, 4, 2) TLF_WS(4, 3, 4, 2)
+#undef TLF_WS
+    }
+  }
 #define TLF_TILE_KG(BN_, BM_, WN_, WM_, NS_, OCC_, KG_)                                     \
   if (!launched && g.bn == BN_ && g.bm == BM_ && g.stages == NS_ && g.occ == OCC_ &&        \
       g.kgroups == KG_ && (g.wn == 0 || g.wn == WN_)) {                                                                   \
@@ -1061,6 +1367,24 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
 
 inline size_t align256(size_t n) { return (n + 255) & ~static_cast<size_t>(255); }
 
+// Row-major int8 [N, K] -> tile order (see the head of this file).  One thread moves one 16-byte
+// atom; rows N .. round_up(N, 32) - 1 of the last group are zero filled.
+__global__ __launch_bounds__(256) void pack_w8_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst,
+                                                      int32_t N, int32_t K, int64_t atoms) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= atoms) return;
+  const int64_t chunk = i >> 6;
+  const int within = static_cast<int>(i & 63);
+  const int kg = within >> 5, r = within & 31;
+  const int chunks_per_group = K / 32;
+  const int64_t group = chunk / chunks_per_group;
+  const int j = static_cast<int>(chunk % chunks_per_group);
+  const int64_t n = group * 32 + r;
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (n < N) v = src[(n * K + (j * 2 + kg) * 16) >> 4];
+  dst[i] = v;
+}
+
 // Projection followed by add-RMSNorm.  A plan that splits K across workgroups ends in the fused
 // reduce + norm kernel; every other plan writes the projection to the head of the workspace and
 // runs the stand-alone add-RMSNorm on it.
@@ -1097,6 +1421,24 @@ inline int check_gemm_args(const void *x, int64_t x_stride, const void *w, const
 }  // namespace tlf
 
 using namespace tlf;
+
+extern "C" size_t tlf_w8a16_packed_bytes(int32_t N, int32_t K) {
+  if (N <= 0 || K <= 0 || K % kBK) return 0;
+  return static_cast<size_t>((N + 31) / 32) * 32 * static_cast<size_t>(K);
+}
+
+extern "C" int tlf_w8a16_pack_weight(const void *wq_rowmajor, void *packed, int32_t N, int32_t K,
+                                     void *stream) {
+  if (!wq_rowmajor || !packed) return TLF_E_NULL;
+  if (N <= 0 || K <= 0 || K % kBK) return TLF_E_SHAPE;
+  if (!aligned16(wq_rowmajor) || !aligned16(packed)) return TLF_E_ALIGN;
+  if (wq_rowmajor == packed) return TLF_E_UNSUPPORTED;  // not in place
+  const int64_t atoms = static_cast<int64_t>(tlf_w8a16_packed_bytes(N, K) / 16);
+  hipLaunchKernelGGL(pack_w8_kernel, dim3(static_cast<unsigned>((atoms + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), static_cast<const uint4 *>(wq_rowmajor),
+                     static_cast<uint4 *>(packed), N, K, atoms);
+  return launch_status();
+}
 
 extern "C" size_t tlf_w8a16_gemm_workspace_bytes(int32_t M, int32_t N, int32_t K) {
   if (M <= 0 || N <= 0 || K <= 0 || K % kBK) return 0;

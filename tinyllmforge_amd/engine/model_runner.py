@@ -50,6 +50,7 @@ class ModelRunner:
                 random_init_(self.model, seed=config.seed, device_fill=big)
             if config.quantization == "w8a16":
                 self.model.quantize_linears_()
+            self.model.pack_linears_()        # int8 weights (quantised here or loaded) into tile order
         finally:
             torch.set_default_dtype(default_dtype)
         self.model.eval()

@@ -3,7 +3,9 @@
 Same class names, weight layout (``[out, in]``, ``nn.Linear`` order) and ``weight_loader``
 protocol as the reference; this build runs one GPU, so the tensor-parallel rank is 0 of 1 and
 there is no all-reduce.  ``quantize_()`` swaps the bf16 weight for an int8 weight plus a
-per-output-channel fp32 scale; ``forward`` then runs the weight-only int8 GEMM.
+per-output-channel fp32 scale; ``forward`` then runs the weight-only int8 GEMM.  On the GPU the int8
+weight is kept in the library's tile order (``ops.pack_w8``, done once by ``pack_()``): ``qweight``
+is the row-major ``[out, in]`` tensor until then, ``qpacked`` the packed one afterwards.
 """
 import torch
 from torch import nn
@@ -28,7 +30,8 @@ class LinearBase(nn.Module):
         self.tp_dim = tp_dim
         self.tp_rank = 0
         self.tp_size = 1
-        self.qweight = None
+        self.qweight = None        # int8 [out, in] row-major (None again once packed)
+        self.qpacked = None        # ops.PackedW8: the same weight in the GEMM kernels' tile order
         self.qscale = None
 
     def _make_params(self, out_features: int, in_features: int, bias: bool):
@@ -43,10 +46,21 @@ class LinearBase(nn.Module):
     def quantize_(self):
         """Replace the bf16 weight by int8 + scale (frees the bf16 copy).  Nothing to do for a layer
         whose int8 weight came from a quantised checkpoint."""
-        if self.qweight is not None:
+        if self.is_quantized:
             return self
         self.qweight, self.qscale = quantize_per_channel(self.weight.data)
         self.weight.data = torch.empty(0, dtype=self.weight.dtype, device=self.weight.device)
+        return self
+
+    @property
+    def is_quantized(self) -> bool:
+        return self.qweight is not None or self.qpacked is not None
+
+    def pack_(self):
+        """Row-major int8 weight -> tile order, on the GPU, once; the row-major copy is dropped."""
+        if self.qpacked is None and self.qweight is not None:
+            self.qpacked = ops.pack_w8(self.qweight)
+            self.qweight = None
         return self
 
     def load_quantized(self, qweight: torch.Tensor, qscale: torch.Tensor):
@@ -78,8 +92,8 @@ class LinearBase(nn.Module):
         self.pending_quantized = False
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        if self.qweight is not None:
-            y = ops.w8a16_linear(x, self.qweight, self.qscale)
+        if self.is_quantized:
+            y = ops.w8a16_linear(x, self.pack_().qpacked, self.qscale)
         else:
             y = ops.bf16_linear(x, self.weight.data)
         if self.bias is not None:
@@ -118,7 +132,7 @@ class MergedColumnParallelLinear(ColumnParallelLinear):
     def quantize_(self):
         """int8 + scale; a gate/up pair is also re-ordered for the fused projection + SiLU-and-mul
         kernel (``ops.gate_up_interleave_index``), which ``forward_silu_mul`` then uses."""
-        if self.qweight is None:
+        if not self.is_quantized:
             super().quantize_()
             self.interleave_()
         return self
@@ -147,7 +161,7 @@ class MergedColumnParallelLinear(ColumnParallelLinear):
     def forward_silu_mul(self, x: torch.Tensor) -> torch.Tensor:
         """``SiluAndMul()(self(x))`` (activation.py:11-14 after linear.py:82-83), fused when quantised."""
         if getattr(self, "interleaved", False):
-            return ops.w8a16_linear_silu_mul(x, self.qweight, self.qscale)
+            return ops.w8a16_linear_silu_mul(x, self.pack_().qpacked, self.qscale)
         return ops.silu_and_mul(super().forward(x))
 
     def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor, loaded_shard_id: int):
@@ -191,8 +205,8 @@ class RowParallelLinear(LinearBase):
         ``norm`` is the ``RMSNorm`` module that follows this projection.  Returns ``(normed, residual)``."""
         if self.bias is not None:
             return norm(self.forward(x), residual)
-        if self.qweight is not None:
-            return ops.linear_add_rms_norm(x, self.qweight, self.qscale, residual, norm.weight.data, norm.eps)
+        if self.is_quantized:
+            return ops.linear_add_rms_norm(x, self.pack_().qpacked, self.qscale, residual, norm.weight.data, norm.eps)
         return ops.linear_add_rms_norm(x, self.weight.data, None, residual, norm.weight.data, norm.eps)
 
     def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor):

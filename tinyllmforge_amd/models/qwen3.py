@@ -170,3 +170,10 @@ class Qwen3ForCausalLM(nn.Module):
             for lin in (layer.self_attn.qkv_proj, layer.self_attn.o_proj, layer.mlp.gate_up_proj, layer.mlp.down_proj):
                 lin.quantize_()
         return self
+
+    def pack_linears_(self):
+        """int8 weights into the GEMM kernels' tile order (on the GPU, once, after loading / quantising)."""
+        for m in self.modules():
+            if hasattr(m, "pack_") and getattr(m, "is_quantized", False):
+                m.pack_()
+        return self

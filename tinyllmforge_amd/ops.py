@@ -208,17 +208,59 @@ def embedding(ids, weight):
 
 
 # ------------------------------------------------------------------ a10
+class PackedW8:
+    """An int8 weight ``[n, k]`` in the tile order the W8A16 kernels read (``tlf_w8a16_pack_weight``):
+    same bytes as the row-major tensor, rows padded to a multiple of 32."""
+    __slots__ = ("data", "n", "k")
+
+    def __init__(self, data: torch.Tensor, n: int, k: int):
+        self.data, self.n, self.k = data, n, k
+
+    @property
+    def shape(self):
+        return (self.n, self.k)
+
+    @property
+    def device(self):
+        return self.data.device
+
+    def data_ptr(self):
+        return self.data.data_ptr()
+
+
+def pack_w8(wq: torch.Tensor) -> PackedW8:
+    """Row-major int8 ``[N, K]`` -> ``PackedW8`` (one pass on the GPU)."""
+    lib = _lib.load()
+    _need(wq, torch.int8, "wq")
+    assert wq.dim() == 2
+    wq = wq.contiguous()
+    N, K = wq.shape
+    nbytes = lib.tlf_w8a16_packed_bytes(N, K)
+    if nbytes == 0:
+        raise _lib.TlfError(f"cannot pack an int8 weight of shape {tuple(wq.shape)} (K % 64 != 0)")
+    out = torch.empty(nbytes, dtype=torch.int8, device=wq.device)
+    check(lib.tlf_w8a16_pack_weight(wq.data_ptr(), out.data_ptr(), N, K, _stream()), "tlf_w8a16_pack_weight")
+    return PackedW8(out, N, K)
+
+
+def _packed(wq) -> PackedW8:
+    """Weights may be given row-major (packed on the fly: convenient for one-off calls) or packed."""
+    return wq if isinstance(wq, PackedW8) else pack_w8(wq)
+
+
 def w8a16_linear(x, wq, scale):
     lib = _lib.load()
-    _need(x, BF16, "x"); _need(wq, torch.int8, "wq"); _need(scale, torch.float32, "scale")
-    assert x.stride(-1) == 1 and wq.is_contiguous()
+    w = _packed(wq)
+    _need(x, BF16, "x"); _need(scale, torch.float32, "scale")
+    assert x.stride(-1) == 1
     x2 = x.reshape(-1, x.shape[-1])
     M, K = x2.shape
-    N = wq.shape[0]
+    N = w.n
+    assert w.k == K and scale.numel() == N
     y = torch.empty(M, N, dtype=BF16, device=x.device)
     nbytes = lib.tlf_w8a16_gemm_workspace_bytes(M, N, K)
     ws = _workspace(nbytes, x.device, "gemm")
-    check(lib.tlf_w8a16_gemm(x2.data_ptr(), x2.stride(0), wq.data_ptr(), scale.data_ptr(), y.data_ptr(),
+    check(lib.tlf_w8a16_gemm(x2.data_ptr(), x2.stride(0), w.data_ptr(), scale.data_ptr(), y.data_ptr(),
                              M, N, K, ws.data_ptr(), ws.numel(), _stream()), "tlf_w8a16_gemm")
     return y.view(*x.shape[:-1], N)
 
@@ -238,13 +280,15 @@ def w8a16_linear_silu_mul(x, wq_interleaved, scale_interleaved):
     """``silu(gate) * up`` of the int8 gate_up projection in one kernel; weight rows interleaved as
     ``gate_up_interleave_index`` says.  Returns ``[..., N / 2]``."""
     lib = _lib.load()
-    _need(x, BF16, "x"); _need(wq_interleaved, torch.int8, "wq"); _need(scale_interleaved, torch.float32, "scale")
-    assert x.stride(-1) == 1 and wq_interleaved.is_contiguous()
+    w = _packed(wq_interleaved)
+    _need(x, BF16, "x"); _need(scale_interleaved, torch.float32, "scale")
+    assert x.stride(-1) == 1
     x2 = x.reshape(-1, x.shape[-1])
     M, K = x2.shape
-    N = wq_interleaved.shape[0]
+    N = w.n
+    assert w.k == K
     y = torch.empty(M, N // 2, dtype=BF16, device=x.device)
-    check(lib.tlf_w8a16_gemm_silu_mul(x2.data_ptr(), x2.stride(0), wq_interleaved.data_ptr(),
+    check(lib.tlf_w8a16_gemm_silu_mul(x2.data_ptr(), x2.stride(0), w.data_ptr(),
                                       scale_interleaved.data_ptr(), y.data_ptr(), M, N, K, _stream()),
           "tlf_w8a16_gemm_silu_mul")
     return y.view(*x.shape[:-1], N // 2)
@@ -284,9 +328,13 @@ def linear_add_rms_norm(x, w, scale, residual, norm_weight, eps):
     or bf16 with ``scale=None``.  Returns ``(normed, new_residual)``, the bits of the two separate calls."""
     lib = _lib.load()
     w8 = scale is not None
-    _need(x, BF16, "x"); _need(w, torch.int8 if w8 else BF16, "w")
-    _need(residual, BF16, "residual"); _need(norm_weight, BF16, "norm_weight")
-    assert x.stride(-1) == 1 and w.is_contiguous() and residual.is_contiguous()
+    if w8:
+        w = _packed(w)
+    else:
+        _need(w, BF16, "w")
+        assert w.is_contiguous()
+    _need(x, BF16, "x"); _need(residual, BF16, "residual"); _need(norm_weight, BF16, "norm_weight")
+    assert x.stride(-1) == 1 and residual.is_contiguous()
     x2 = x.reshape(-1, x.shape[-1])
     M, K = x2.shape
     N = w.shape[0]
