@@ -499,8 +499,8 @@ void gemm_dlds_kernel(const GemmParams p) {
 // W-streaming kernel for decode-size batches, int8 weights in tile order.
 //
 // At these sizes every weight byte is used once per token tile and the kernel lives or dies by how
-// the 256 CUs pull the weight matrix out of HBM.  A workgroup owns 128 channels and all tokens.
-// Its 4 x KG compute waves are 4 side by side along N times KG along K: wave (n, kh) owns one
+// the 256 CUs pull the weight matrix out of HBM.  A workgroup owns 32 COLS channels and all tokens.
+// Its COLS x KG compute waves are COLS side by side along N times KG along K: wave (n, kh) owns one
 // 32-row group of W for the kh-th part of the workgroup's K range and streams it global -> registers:
 // one contiguous run, 1 KiB per load instruction, PF K-tiles (2 KiB each) in flight per wave, no LDS
 // and no workgroup barrier on the weight side; each lane's 16 bytes are its MFMA A operand after the
@@ -510,11 +510,13 @@ void gemm_dlds_kernel(const GemmParams p) {
 // one barrier per step hands a stage over.  KG = 2 puts two compute waves on every SIMD, which take
 // turns in the matrix pipe while the other one waits for LDS or converts; their accumulators are
 // added through LDS at the end.  Accumulator layout and epilogue are those of the tiled kernel.
-constexpr int kWsCols = 4;  // compute waves side by side along N (128 channels per workgroup)
-
-template <int TM, int NS, int PF, int KG>
-__global__ __launch_bounds__((kWsCols * KG + 1) * 64) __attribute__((amdgpu_waves_per_eu(1, KG + 1)))
+// COLS = compute waves side by side along N (3 or 4: 96 or 128 channels per workgroup; the host picks
+// the width whose workgroup count fills the 256 CUs best - a kernel that is bound by HBM needs every
+// CU pulling: 24576 channels are 192 workgroups of 128 but 256 of 96).
+template <int TM, int NS, int PF, int KG, int COLS>
+__global__ __launch_bounds__((COLS * KG + 1) * 64) __attribute__((amdgpu_waves_per_eu(1, (COLS * KG + 4) / 4)))
 void gemm_wstream_kernel(const GemmParams p) {
+  constexpr int kWsCols = COLS;
   constexpr int BM = TM * 32;
   constexpr int kCompute = kWsCols * KG;
   constexpr int kXBytes = BM * 128;        // one x tile: BM rows of 64 bf16
@@ -983,6 +985,7 @@ __global__ __launch_bounds__(512) void skinny_gemm_kernel(const GemmParams p) {
 //   TLF_GEMM_WSTREAM_M="lo,hi"  token range served by the W-streaming kernel ("0,0": never)
 //   TLF_GEMM_WSTREAM_SPLITS     its split of K across workgroups
 //   TLF_GEMM_WSTREAM_KG         its K parts inside a workgroup (1 or 2)
+//   TLF_GEMM_WSTREAM_COLS       its workgroup width in 32-channel groups (3 or 4)
 //   TLF_GEMM_WSTREAM_FORCE=1    take it for every shape in its token range, not only where it measured faster
 struct GemmTuning {
   bool has_plan = false;
@@ -994,6 +997,7 @@ struct GemmTuning {
   int ws_splits = 0;                               // forced split of K for it
   int ws_kg = 0;                                   // forced K parts per workgroup (1 or 2)
   bool ws_force = false;                           // take it for every shape in its token range
+  int ws_cols = 0;                                 // forced workgroup width in 32-channel groups (3 or 4)
 };
 
 inline const GemmTuning &gemm_tuning() {
@@ -1024,6 +1028,7 @@ inline const GemmTuning &gemm_tuning() {
     }
     if (const char *e = getenv("TLF_GEMM_WSTREAM_SPLITS")) g.ws_splits = atoi(e) > 0 ? atoi(e) : 0;
     if (const char *e = getenv("TLF_GEMM_WSTREAM_FORCE")) g.ws_force = atoi(e) != 0;
+    if (const char *e = getenv("TLF_GEMM_WSTREAM_COLS")) g.ws_cols = atoi(e);
     if (const char *e = getenv("TLF_GEMM_WSTREAM_KG")) g.ws_kg = atoi(e) == 1 || atoi(e) == 2 ? atoi(e) : 0;
     return g;
   }();
@@ -1077,7 +1082,12 @@ struct GemmPlan {
 inline bool plan_wstream(int M, int N, int K, int act, GemmPlan &g) {
   const GemmTuning &t = gemm_tuning();
   if (t.has_plan || M < t.ws_min_m || M > t.ws_max_m || M < 1 || act == 2) return false;
-  const int n_wg = (N + 127) / 128;
+  // 128 or 96 channels per workgroup: whichever count of workgroups fills whole rounds of 256 CUs better
+  auto fill = [](int wgs) { return static_cast<double>(wgs) / ((wgs + 255) / 256 * 256); };
+  int cols = 4;
+  if (N >= 256 * 96 && fill((N + 95) / 96) > fill((N + 127) / 128) + 0.1) cols = 3;
+  if (t.ws_cols == 3 || t.ws_cols == 4) cols = t.ws_cols;
+  const int n_wg = (N + cols * 32 - 1) / (cols * 32);
   const int ktiles = K / kBK;
   int splits = 1;
   // Measured against the tiled plans on the Qwen3-8B projections with cold weights: a wide N (gate_up)
@@ -1098,7 +1108,7 @@ inline bool plan_wstream(int M, int N, int K, int act, GemmPlan &g) {
   const int kt_per = (ktiles + splits - 1) / splits;
   const int tm = (M + 31) / 32;
   g.wstream = true;
-  g.bn = 128;
+  g.bn = cols * 32;
   g.bm = tm * 32;
   int kg = ktiles % 2 == 0 && kt_per >= 4 ? 2 : 1;
   if (t.ws_kg && (t.ws_kg == 1 || ktiles % 2 == 0)) kg = t.ws_kg;
@@ -1292,15 +1302,18 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   if constexpr (W8) {
     if (g.wstream) {
       const dim3 wgrid(p.n_tiles, g.splits);
-#define TLF_WS(TM_, NS_, PF_, KG_)                                                                  \
-  if (!launched && g.bm == TM_ * 32 && g.kgroups == KG_) {                                          \
+#define TLF_WS(TM_, NS_, PF_, KG_, COLS_)                                                           \
+  if (!launched && g.bm == TM_ * 32 && g.kgroups == KG_ && g.bn == COLS_ * 32) {                    \
     if (!dry)                                                                                       \
-      hipLaunchKernelGGL((gemm_wstream_kernel<TM_, NS_, PF_, KG_>), wgrid,                          \
-                         dim3((kWsCols * KG_ + 1) * 64), 0, stream, p);                             \
+      hipLaunchKernelGGL((gemm_wstream_kernel<TM_, NS_, PF_, KG_, COLS_>), wgrid,                   \
+                         dim3((COLS_ * KG_ + 1) * 64), 0, stream, p);                               \
     launched = true;                                                                                \
   }
-      TLF_WS(1, 4, 8, 1) TLF_WS(2, 4, 8, 1) TLF_WS(3, 4, 8, 1) TLF_WS(4, 4, 8, 1)
-      TLF_WS(1, 4, 4, 2) TLF_WS(2, 4, 4, 2) TLF_WS(3, 3, 4, 2) TLF_WS(4, 3, 4, 2)
+      // registers per wave: 9 waves (4 x 2 + 1) leave 168, so the tall tiles keep 4 weight tiles in flight there
+      TLF_WS(1, 4, 8, 1, 4) TLF_WS(2, 4, 8, 1, 4) TLF_WS(3, 4, 8, 1, 4) TLF_WS(4, 4, 8, 1, 4)
+      TLF_WS(1, 4, 8, 2, 4) TLF_WS(2, 4, 8, 2, 4) TLF_WS(3, 3, 4, 2, 4) TLF_WS(4, 3, 4, 2, 4)
+      TLF_WS(1, 4, 8, 1, 3) TLF_WS(2, 4, 8, 1, 3) TLF_WS(3, 4, 8, 1, 3) TLF_WS(4, 4, 8, 1, 3)
+      TLF_WS(1, 4, 8, 2, 3) TLF_WS(2, 4, 8, 2, 3) TLF_WS(3, 3, 8, 2, 3) TLF_WS(4, 3, 8, 2, 3)
 #undef TLF_WS
     }
   }
