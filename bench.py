@@ -52,7 +52,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=0,
                     help="engine steps that steps/ms_per_step describe (0 = all); value is always the whole job")
     ap.add_argument("--warmup", type=int, default=1, help="warm-up generate() calls before the timed run")
-    ap.add_argument("--workload", default="e2e", choices=["e2e", "decode_attn", "gemm", "c5", "all"])
+    ap.add_argument("--workload", default="e2e", choices=["e2e", "decode_attn", "gemm", "prefill_attn", "c5", "all"])
     ap.add_argument("--attn-steps", type=int, default=200, help="timed launches of the decode-attention microbench")
     ap.add_argument("--num-seqs", type=int, default=256)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -281,6 +281,53 @@ def cpu_baseline_gemm(budget_s=20.0):
                        f"{spent:.1f} s of CPU oracle time")
 
 
+# ----------------------------------------------------------------------------- prefill attention microbench
+def bench_prefill_attn(args):
+    """Varlen causal prefill attention at the 8B shape (32 / 8 heads, packed bf16 K/V) and the 32B shape
+    (64 / 8 heads, paged e4m3 rows, optionally behind a cached prefix).  flops = 4 Hq Dh sum(len^2 / 2 +
+    len * cached); frac against the dense bf16 MFMA peak."""
+    import torch
+    from tinyllmforge_amd import ops as P
+    torch.manual_seed(0)
+    dev, dh, bs = "cuda", 128, 256
+    rows = []
+
+    def run(name, lens, hq, hkv, fp8=False, cached=0):
+        S = sum(lens)
+        q = torch.randn(S, hq, dh, device=dev).to(torch.bfloat16)
+        cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=dev)
+        flops = sum(4.0 * hq * dh * (l * l / 2 + l * cached) for l in lens)
+        if not fp8:
+            k = torch.randn(S, hkv, dh, device=dev).to(torch.bfloat16)
+            v = torch.randn(S, hkv, dh, device=dev).to(torch.bfloat16)
+            f = lambda: P.varlen_prefill_attention(q, k, v, cu, cu, max(lens), 1 / math.sqrt(dh))
+        else:
+            klens = [l + cached for l in lens]
+            nb = [(l + bs - 1) // bs for l in klens]
+            kc = (torch.randn(sum(nb), bs, hkv, dh, device=dev) * 0.5).to(torch.float8_e4m3fn)
+            vc = (torch.randn(sum(nb), bs, hkv, dh, device=dev) * 0.5).to(torch.float8_e4m3fn)
+            bt = torch.full((len(lens), max(nb)), -1, dtype=torch.int32)
+            o = 0
+            for i, n in enumerate(nb):
+                bt[i, :n] = torch.arange(o, o + n)
+                o += n
+            bt = bt.to(dev)
+            cuk = torch.tensor([0] + list(torch.tensor(klens).cumsum(0)), dtype=torch.int32, device=dev)
+            ksc, vsc = torch.full((hkv,), 0.02, device=dev), torch.full((hkv,), 0.02, device=dev)
+            f = lambda: P.varlen_prefill_attention(q, kc, vc, cu, cuk, max(lens), 1 / math.sqrt(dh), block_tables=bt,
+                                                   k_scale=ksc, v_scale=vsc)
+        sec = time_graph(f, 5, 5) * 1e-3
+        rows.append(dict(case=name, tokens=S, us=round(sec * 1e6, 1), TFLOPs=round(flops / sec / 1e12, 1),
+                         frac=round(flops / sec / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)))
+
+    run("8B shape, bf16 rows, 16 x 1024 tokens", [1024] * 16, 32, 8)
+    run("8B shape, bf16 rows, 28 x 560 tokens", [560] * 28, 32, 8)
+    run("8B shape, bf16 rows, 4 x 4096 tokens", [4096] * 4, 32, 8)
+    run("32B shape, e4m3 rows (paged), 2 x 8192 tokens", [8192] * 2, 64, 8, fp8=True)
+    run("32B shape, e4m3 rows (paged), 3 x 4096 tokens behind 1024 cached", [4096] * 3, 64, 8, fp8=True, cached=1024)
+    return rows
+
+
 # ----------------------------------------------------------------------------- config 5 (32B shape, fp8 KV, shared prefixes)
 def bench_c5(args):
     """BASELINE.json configs[4]: Qwen3-32B-shaped decoder, W8A16 linears, e4m3 KV cache with per-head scales,
@@ -458,6 +505,19 @@ def main():
                                    "Qwen3-8B projection shapes, M = 1 ... 8192, random normal x, random int8 W"},
             "roofline": roofline, "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline_gemm(),
             "extra": extra}))
+        return
+    if args.workload == "prefill_attn":   # its own line: the prefill-attention microbench
+        rows = bench_prefill_attn(args)
+        extra["prefill_attn"] = rows
+        best = max(rows, key=lambda r: r["TFLOPs"])
+        print(json.dumps({
+            "metric": "varlen causal prefill attention TFLOP/s vs bf16 MFMA peak", "value": best["TFLOPs"], "unit": "TFLOP/s",
+            "n_gpus": 1, "steps": 25, "warmup": 6, "ms_per_step": round(best["us"] * 1e-3, 4), "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "prefill attention microbench: " + best["case"]},
+            "roofline": {"bound": "mfma", "achieved": best["TFLOPs"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                         "frac": best["frac"], "traffic": None, "kernel": "prefill_attn_kernel"},
+            "cpu_baseline": None, "extra": extra}))
         return
     if args.workload == "decode_attn":
         cpu = None if args.no_cpu_baseline else cpu_baseline_decode(attn["case"])

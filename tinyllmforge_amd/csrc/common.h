@@ -69,6 +69,13 @@ __device__ __forceinline__ uint4 pack8(const float (&f)[8]) {
   return p;
 }
 
+// Four e4m3 values (one dword) -> four bf16, exact: v_cvt_scalef32_pk_bf16_fp8 converts a pair per
+// instruction (scale 1.0), half the vector-ALU work of going through fp32.
+__device__ __forceinline__ void fp8x4_to_bf16x4(unsigned int w, unsigned int &lo, unsigned int &hi) {
+  lo = __builtin_bit_cast(unsigned int, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, false));
+  hi = __builtin_bit_cast(unsigned int, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(w, 1.0f, true));
+}
+
 // 128-bit load with the non-temporal hint: data that is read once (KV-cache rows,
 // weights at small batch) should not displace L2 / Infinity Cache lines; on MI355X a
 // read-only stream is ~10% faster with it (measured: 7.1 vs 6.3 TB/s).

@@ -78,16 +78,10 @@ __device__ __forceinline__ shortx4 lds_read_tr16_b64(const unsigned short *p) {
 }
 
 __device__ __forceinline__ void fp8x16_to_bf16x16(const uint4 &in, uint4 &lo, uint4 &hi) {
-  auto cv = [](unsigned int w, unsigned int &a, unsigned int &b) {
-    const auto f0 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w), false);
-    const auto f1 = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w), true);
-    a = pack_bf16x2(f0[0], f0[1]);
-    b = pack_bf16x2(f1[0], f1[1]);
-  };
-  cv(in.x, lo.x, lo.y);
-  cv(in.y, lo.z, lo.w);
-  cv(in.z, hi.x, hi.y);
-  cv(in.w, hi.z, hi.w);
+  fp8x4_to_bf16x4(in.x, lo.x, lo.y);
+  fp8x4_to_bf16x4(in.y, lo.z, lo.w);
+  fp8x4_to_bf16x4(in.z, hi.x, hi.y);
+  fp8x4_to_bf16x4(in.w, hi.z, hi.w);
 }
 
 // One tile's worth of global data of one wave: 16 tokens x 128 dims of K and V
