@@ -292,30 +292,33 @@ void paged_decode_kernel(const DecodeParams p) {
         const float m_new = fmaxf(m_run, mt);
         // -inf only while every token so far sat in a skipped block: keep the exponents finite
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = exp2f(m_run - m_use);
-        float psum = 0.f;
-        bf16x4 pb, pl;
+        // raw v_exp_f32: results below 2^-126 (which the library routine would denormalise) weigh nothing here
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+        float pv[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float pv = exp2f(sv[i] - m_use);
-          psum += pv;
-          pb[i] = static_cast<__bf16>(pv);
-          pl[i] = static_cast<__bf16>(pv - static_cast<float>(pb[i]));
-        }
-        l_run = l_run * alpha + psum;
+        for (int i = 0; i < 4; ++i) pv[i] = __builtin_amdgcn_exp2f(sv[i] - m_use);
+        l_run = l_run * alpha + ((pv[0] + pv[1]) + (pv[2] + pv[3]));
         m_run = m_new;
-        const shortx4 pbs = __builtin_bit_cast(shortx4, pb);
-        const shortx4 pls = __builtin_bit_cast(shortx4, pl);
-        // the running max rarely moves after the first tiles: skip the 32 multiplies then (wave-uniform)
-        const bool rescale = __any(alpha != 1.0f);
+        // P as a bf16 hi + lo pair, converted two at a time
+        const unsigned int hi01 = pack_bf16x2(pv[0], pv[1]), hi23 = pack_bf16x2(pv[2], pv[3]);
+        const unsigned int lo01 = pack_bf16x2(pv[0] - __uint_as_float(hi01 << 16), pv[1] - __uint_as_float(hi01 & 0xffff0000u));
+        const unsigned int lo23 = pack_bf16x2(pv[2] - __uint_as_float(hi23 << 16), pv[3] - __uint_as_float(hi23 & 0xffff0000u));
+        const shortx4 pbs = __builtin_bit_cast(shortx4, make_uint2(hi01, hi23));
+        const shortx4 pls = __builtin_bit_cast(shortx4, make_uint2(lo01, lo23));
+        // the running max rarely moves after the first tiles: skip the 32 multiplies then.  The branch is
+        // wave-uniform and must stay a branch (the empty asm keeps the compiler from turning it into 32
+        // multiplies and 32 selects on every tile).
+        if (__any(alpha != 1.0f)) {
+          asm volatile("" ::);
+#pragma unroll
+          for (int d = 0; d < 8; ++d)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[d][i] *= alpha;
+        }
 #pragma unroll
         for (int d = 0; d < 8; ++d) {
           // A = V^T fragment: lane (dim = d*16 + n, g) <- tokens g*4 + 0..3 (transpose read)
           const shortx4 vf = lds_read_tr16_b64(&Vs[g * 4 + (n >> 2)][d * 16 + (n & 3) * 4]);
-          if (rescale) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[d][i] *= alpha;
-          }
           acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pbs, acc[d], 0, 0, 0);
           acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pls, acc[d], 0, 0, 0);
         }
