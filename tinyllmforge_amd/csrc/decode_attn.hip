@@ -41,7 +41,11 @@ namespace tlf {
 
 constexpr int kDh = 128;
 constexpr int kTile = 16;             // tokens per tile
-constexpr int kLdsRow = kDh + 8;      // padded LDS row (elements): 272 B, shifts rows by 4 banks
+// Padded LDS rows (elements).  LDS has 32 banks of 4 bytes.  K rows are read 16 bytes per lane by 8 lanes of 8
+// consecutive rows at a time: a 272-byte row shifts each row by 4 banks.  V rows are read transposed, 8 bytes
+// per lane, 4 lanes per row and 4 rows at a time: a 288-byte row shifts each row by 8 banks.
+constexpr int kLdsRowK = kDh + 8;
+constexpr int kLdsRowV = kDh + 16;
 constexpr int kMaxBatch = 1024;       // sequences per call (prefix table lives in LDS)
 constexpr int kMinTiles = 4;          // smallest share of a workgroup, in tiles
 constexpr int kMaxGrid = 1024;        // workspace is sized for this many workgroups
@@ -84,6 +88,18 @@ __device__ __forceinline__ void fp8x16_to_bf16x16(const uint4 &in, uint4 &lo, ui
   fp8x4_to_bf16x4(in.w, hi.z, hi.w);
 }
 
+// Head dimension held by LDS column c of a K or V tile.  bf16 rows are stored as they come.  e4m3 rows are
+// stored with their 16-byte halves regrouped (columns 0..63: dims 16 j + 0..7, columns 64..127: dims 16 j + 8..15)
+// so that the conversion's LDS writes are conflict free; the first product sums over columns (q is read with the
+// same permutation) and the second product's output rows are columns (mapped back when written).  Runs of 8
+// columns stay runs of 8 dims.
+template <bool KV8>
+__device__ __forceinline__ int lds_col_dim(int c) {
+  if (!KV8) return c;
+  const int j = (c >> 3) & 7;
+  return j * 16 + (c >= 64 ? 8 : 0) + (c & 7);
+}
+
 // One tile's worth of global data of one wave: 16 tokens x 128 dims of K and V
 // (4 + 4 128-bit loads per lane for bf16, 2 + 2 for e4m3).
 template <bool KV8>
@@ -96,11 +112,20 @@ struct TileRegs {
 
 // PF = tiles in flight per wave (register prefetch depth).  PF == 1 fits 128 VGPRs, i.e. two
 // 8-wave workgroups per CU; deeper prefetch runs one workgroup per CU with up to 256 VGPRs.
-template <int NW, bool KV8, int PF>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(PF == 1 ? 4 : 2, 4)))
+//
+// TS = 16-token tiles per loop trip.  bf16 rows: 1.  e4m3 rows: 2, so that a trip moves the same bytes per wave
+// as a bf16 trip does (a wave with 4 KB in flight per trip does not cover the latency of its own loads), and
+// the 32 tokens share one softmax step (one pair of cross-lane exchanges, one rescale) and feed the second
+// product through v_mfma_f32_16x16x32_bf16: the K index inside an MFMA is only a summation label, so label
+// g*8 + j stands for token g*4 + j%4 of tile j/4, which is where the first product left the scores.
+template <int NW, bool KV8, int PF, int TS>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(PF == 1 && TS == 1 ? 4 : 2, 4)))
 void paged_decode_kernel(const DecodeParams p) {
   constexpr int kThreads = NW * 64;
-  __shared__ __attribute__((aligned(16))) unsigned short lds[NW][2][kTile][kLdsRow];
+  constexpr int kTrip = TS * kTile;  // tokens per loop trip
+  static_assert(TS == 1 || TS == 2, "one or two tiles per trip");
+  __shared__ __attribute__((aligned(16))) unsigned short lds_k[NW][kTrip][kLdsRowK];
+  __shared__ __attribute__((aligned(16))) unsigned short lds_v[NW][kTrip][kLdsRowV];
   __shared__ int s_prefix[kMaxBatch + 1];  // tiles before sequence b
   __shared__ int s_wave_tot[16];
   __shared__ int s_start_b;
@@ -167,8 +192,8 @@ void paged_decode_kernel(const DecodeParams p) {
   __syncthreads();
 
   const int64_t row_elems = static_cast<int64_t>(p.num_kv_heads) * kDh;
-  unsigned short(*Ks)[kLdsRow] = lds[w][0];
-  unsigned short(*Vs)[kLdsRow] = lds[w][1];
+  unsigned short(*Ks)[kLdsRowK] = lds_k[w];
+  unsigned short(*Vs)[kLdsRowV] = lds_v[w];
   const float kscale = KV8 ? p.k_scale[w] : 1.0f;
   const float vscale = KV8 ? p.v_scale[w] : 1.0f;
   const float scale_log2 = p.scale_log2 * kscale;
@@ -192,47 +217,76 @@ void paged_decode_kernel(const DecodeParams p) {
       for (int c = 0; c < 4; ++c) {
         Pack16 t;
         t.u = make_uint4(0, 0, 0, 0);
-        if (head_ok) t.u = *reinterpret_cast<const uint4 *>(qp + c * 32 + g * 8);
+        if (head_ok) t.u = *reinterpret_cast<const uint4 *>(qp + lds_col_dim<KV8>(c * 32 + g * 8));
         qf[c] = t.v;
       }
     }
+    // Block-table entries: lane i holds entry bt_base + i (64 blocks at a time), and a tile's entry is read out of
+    // that register by lane index.  A per-tile fetch would sit in the in-order load queue between the tile loads,
+    // and waiting for it would drain the tile loads issued before it.
     const int32_t *bt = p.block_tables + b * p.bt_stride;
+    int bt_base = t_begin / p.block_size;
+    int bt_vec = bt[min(bt_base + lane, p.max_blocks - 1)];
+    auto block_of = [&](int tok) {  // tok is wave-uniform and not before the tokens asked for earlier
+      const int bi = __builtin_amdgcn_readfirstlane(tok / p.block_size);
+      if (bi - bt_base >= 64) {  // uniform, once per 64 blocks
+        bt_base = bi;
+        bt_vec = bt[min(bt_base + lane, p.max_blocks - 1)];
+      }
+      return __builtin_amdgcn_readlane(bt_vec, bi - bt_base);
+    };
 
-    // Issue the loads of the tile starting at token t0 (a tile never straddles a block);
-    // blk is its block-table entry, fetched one tile earlier so that its latency is hidden.
-    auto load_tile = [&](int t0, int64_t blk, TileRegs<KV8> &r) {
+    // Issue the loads of the tile starting at token t0 (a tile never straddles a block); blk is its
+    // block-table entry.  The address is a wave-uniform base (the tile's first row) plus a per-lane byte
+    // offset that never changes: no vector-ALU address arithmetic per tile.  A tile that lies wholly inside
+    // the segment (all but a segment's last) loads without predicates.
+    // bf16: 4 tokens x 16 chunks of 8 elements per instruction; e4m3: 8 tokens x 8 chunks of 16
+    const unsigned int lane_off = KV8 ? static_cast<unsigned int>((lane >> 3) * row_elems + w * kDh + (lane & 7) * 16)
+                                      : static_cast<unsigned int>((g * row_elems + w * kDh + n * 8) * 2);
+    const unsigned int load_stride = static_cast<unsigned int>(KV8 ? 8 * row_elems : 4 * row_elems * 2);
+    auto load_tile = [&](int t0, int blk, TileRegs<KV8> &r) {
       const int bi = t0 / p.block_size;
       const bool ok = blk >= 0 && blk < p.num_cache_blocks;
-      const int64_t tok0 = (ok ? blk : 0) * p.block_size + (t0 - bi * p.block_size);
+      const int64_t tok0 = static_cast<int64_t>(ok ? blk : 0) * p.block_size + (t0 - bi * p.block_size);
+      const int64_t base = tok0 * row_elems * (KV8 ? 1 : 2);
+      const unsigned char *kb = p.k_cache + base, *vb = p.v_cache + base;
       r.ok = ok;
+      if (ok && t0 + kTile <= t_end) {  // uniform
 #pragma unroll
-      for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
-        // bf16: 4 tokens x 16 chunks of 8 elements per instruction; e4m3: 8 tokens x 8 chunks of 16
-        const int tt = KV8 ? i * 8 + (lane >> 3) : i * 4 + g;
-        const int64_t off = KV8 ? (tok0 + tt) * row_elems + w * kDh + (lane & 7) * 16
-                                : ((tok0 + tt) * row_elems + w * kDh + n * 8) * 2;
-        const bool valid = ok && (t0 + tt) < t_end;
-        r.k[i] = make_uint4(0, 0, 0, 0);
-        r.v[i] = make_uint4(0, 0, 0, 0);
-        if (valid) {
-          r.k[i] = load_nt_u4(p.k_cache + off);
-          r.v[i] = load_nt_u4(p.v_cache + off);
+        for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
+          r.k[i] = load_nt_u4(kb + (lane_off + i * load_stride));
+          r.v[i] = load_nt_u4(vb + (lane_off + i * load_stride));
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
+          const int tt = KV8 ? i * 8 + (lane >> 3) : i * 4 + g;
+          r.k[i] = make_uint4(0, 0, 0, 0);
+          r.v[i] = make_uint4(0, 0, 0, 0);
+          if (ok && (t0 + tt) < t_end) {
+            r.k[i] = load_nt_u4(kb + (lane_off + i * load_stride));
+            r.v[i] = load_nt_u4(vb + (lane_off + i * load_stride));
+          }
         }
       }
     };
-    auto store_tile = [&](const TileRegs<KV8> &r) {
+    auto store_tile = [&](const TileRegs<KV8> &r, int row0) {
+      unsigned short(*Ks)[kLdsRowK] = lds_k[w] + row0;
+      unsigned short(*Vs)[kLdsRowV] = lds_v[w] + row0;
 #pragma unroll
       for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
         if (KV8) {
+          // a lane holds dims 16 c .. 16 c + 15 (c = lane % 8): the first eight go to LDS columns 8 c ..,
+          // the other eight to columns 64 + 8 c .., so that 8 lanes write 128 contiguous bytes (lds_col_dim)
           const int tt = i * 8 + (lane >> 3);
-          const int ch = (lane & 7) * 16;
+          const int ch = (lane & 7) * 8;
           uint4 lo, hi;
           fp8x16_to_bf16x16(r.k[i], lo, hi);
           *reinterpret_cast<uint4 *>(&Ks[tt][ch]) = lo;
-          *reinterpret_cast<uint4 *>(&Ks[tt][ch + 8]) = hi;
+          *reinterpret_cast<uint4 *>(&Ks[tt][64 + ch]) = hi;
           fp8x16_to_bf16x16(r.v[i], lo, hi);
           *reinterpret_cast<uint4 *>(&Vs[tt][ch]) = lo;
-          *reinterpret_cast<uint4 *>(&Vs[tt][ch + 8]) = hi;
+          *reinterpret_cast<uint4 *>(&Vs[tt][64 + ch]) = hi;
         } else {
           *reinterpret_cast<uint4 *>(&Ks[i * 4 + g][n * 8]) = r.k[i];
           *reinterpret_cast<uint4 *>(&Vs[i * 4 + g][n * 8]) = r.v[i];
@@ -246,47 +300,66 @@ void paged_decode_kernel(const DecodeParams p) {
     float m_run = -INFINITY;  // running max (log2 domain), identical in the 4 lanes of a head
     float l_run = 0.f;        // this lane's share of the running sum
 
-    // PF tiles are kept in flight: tile j of a group of PF lives in regs[j]; block-table entries
-    // are fetched PF tiles before the loads that need them.
-    TileRegs<KV8> regs[PF];
-    int next_blk[PF];
+    // PF trips are kept in flight: tile h of trip j of a group of PF lives in regs[j][h].
+    TileRegs<KV8> regs[PF][TS];
 #pragma unroll
-    for (int j = 0; j < PF; ++j) {
-      const int tj = t_begin + j * kTile;
-      if (tj < t_end) load_tile(tj, bt[tj / p.block_size], regs[j]);
-      next_blk[j] = bt[min(tj + PF * kTile, t_end - 1) / p.block_size];
-    }
-    for (int tg = t_begin; tg < t_end; tg += PF * kTile) {
+    for (int j = 0; j < PF; ++j)
+#pragma unroll
+      for (int h = 0; h < TS; ++h) {
+        const int tj = t_begin + j * kTrip + h * kTile;
+        regs[j][h].ok = false;
+        if (tj < t_end) load_tile(tj, block_of(tj), regs[j][h]);
+      }
+    for (int tg = t_begin; tg < t_end; tg += PF * kTrip) {
 #pragma unroll
       for (int j = 0; j < PF; ++j) {
-        const int t0 = tg + j * kTile;
+        const int t0 = tg + j * kTrip;
         if (t0 >= t_end) break;  // uniform
-        wave_lds_fence();  // previous tile's LDS reads are done
-        store_tile(regs[j]);
+        wave_lds_fence();  // previous trip's LDS reads are done
+        bool tile_ok[TS];
+#pragma unroll
+        for (int h = 0; h < TS; ++h) {
+          // a tile past the end of the segment (second tile of the last trip) was never loaded: zeros, masked below
+          if (t0 + h * kTile >= t_end) {
+#pragma unroll
+            for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
+              regs[j][h].k[i] = make_uint4(0, 0, 0, 0);
+              regs[j][h].v[i] = make_uint4(0, 0, 0, 0);
+            }
+            regs[j][h].ok = false;
+          }
+          store_tile(regs[j][h], h * kTile);
+          tile_ok[h] = regs[j][h].ok;
+        }
         wave_lds_fence();
-        const bool tile_ok = regs[j].ok;
-        const int tn = t0 + PF * kTile;
-        if (tn < t_end) {
-          load_tile(tn, next_blk[j], regs[j]);
-          next_blk[j] = bt[min(tn + PF * kTile, t_end - 1) / p.block_size];
+#pragma unroll
+        for (int h = 0; h < TS; ++h) {
+          const int tn = t0 + PF * kTrip + h * kTile;
+          if (tn < t_end) load_tile(tn, block_of(tn), regs[j][h]);
         }
 
-        // S^T = K . Q^T : lane (n, g) gets tokens g*4 + i of head n
-        floatx4 s = floatx4{0.f, 0.f, 0.f, 0.f};
+        // S^T = K . Q^T : lane (n, g) gets tokens g*4 + i of head n, for each tile of the trip
+        floatx4 s[TS];
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
-          Pack16 a;
-          a.u = *reinterpret_cast<const uint4 *>(&Ks[n][c * 32 + g * 8]);
-          s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[c], s, 0, 0, 0);
-        }
-        float sv[4];
+        for (int h = 0; h < TS; ++h) s[h] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+#pragma unroll
+          for (int h = 0; h < TS; ++h) {
+            Pack16 a;
+            a.u = *reinterpret_cast<const uint4 *>(&Ks[h * kTile + n][c * 32 + g * 8]);
+            s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[c], s[h], 0, 0, 0);
+          }
+        float sv[TS][4];
         float mt = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const bool valid = tile_ok && (t0 + g * 4 + i) < t_end;
-          sv[i] = valid ? s[i] * scale_log2 : -INFINITY;
-          mt = fmaxf(mt, sv[i]);
-        }
+        for (int h = 0; h < TS; ++h)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            const bool valid = tile_ok[h] && (t0 + h * kTile + g * 4 + i) < t_end;
+            sv[h][i] = valid ? s[h][i] * scale_log2 : -INFINITY;
+            mt = fmaxf(mt, sv[h][i]);
+          }
         mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
         mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
         const float m_new = fmaxf(m_run, mt);
@@ -294,20 +367,29 @@ void paged_decode_kernel(const DecodeParams p) {
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
         // raw v_exp_f32: results below 2^-126 (which the library routine would denormalise) weigh nothing here
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
-        float pv[4];
+        float pv[TS][4];
+        float psum = 0.f;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) pv[i] = __builtin_amdgcn_exp2f(sv[i] - m_use);
-        l_run = l_run * alpha + ((pv[0] + pv[1]) + (pv[2] + pv[3]));
+        for (int h = 0; h < TS; ++h) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) pv[h][i] = __builtin_amdgcn_exp2f(sv[h][i] - m_use);
+          psum += (pv[h][0] + pv[h][1]) + (pv[h][2] + pv[h][3]);
+        }
+        l_run = l_run * alpha + psum;
         m_run = m_new;
         // P as a bf16 hi + lo pair, converted two at a time
-        const unsigned int hi01 = pack_bf16x2(pv[0], pv[1]), hi23 = pack_bf16x2(pv[2], pv[3]);
-        const unsigned int lo01 = pack_bf16x2(pv[0] - __uint_as_float(hi01 << 16), pv[1] - __uint_as_float(hi01 & 0xffff0000u));
-        const unsigned int lo23 = pack_bf16x2(pv[2] - __uint_as_float(hi23 << 16), pv[3] - __uint_as_float(hi23 & 0xffff0000u));
-        const shortx4 pbs = __builtin_bit_cast(shortx4, make_uint2(hi01, hi23));
-        const shortx4 pls = __builtin_bit_cast(shortx4, make_uint2(lo01, lo23));
+        unsigned int hi[TS][2], lo[TS][2];
+#pragma unroll
+        for (int h = 0; h < TS; ++h)
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            hi[h][e] = pack_bf16x2(pv[h][2 * e], pv[h][2 * e + 1]);
+            lo[h][e] = pack_bf16x2(pv[h][2 * e] - __uint_as_float(hi[h][e] << 16),
+                                   pv[h][2 * e + 1] - __uint_as_float(hi[h][e] & 0xffff0000u));
+          }
         // the running max rarely moves after the first tiles: skip the 32 multiplies then.  The branch is
         // wave-uniform and must stay a branch (the empty asm keeps the compiler from turning it into 32
-        // multiplies and 32 selects on every tile).
+        // multiplies and 32 selects on every trip).
         if (__any(alpha != 1.0f)) {
           asm volatile("" ::);
 #pragma unroll
@@ -315,12 +397,32 @@ void paged_decode_kernel(const DecodeParams p) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) acc[d][i] *= alpha;
         }
+        if constexpr (TS == 1) {
+          const shortx4 pbs = __builtin_bit_cast(shortx4, make_uint2(hi[0][0], hi[0][1]));
+          const shortx4 pls = __builtin_bit_cast(shortx4, make_uint2(lo[0][0], lo[0][1]));
 #pragma unroll
-        for (int d = 0; d < 8; ++d) {
-          // A = V^T fragment: lane (dim = d*16 + n, g) <- tokens g*4 + 0..3 (transpose read)
-          const shortx4 vf = lds_read_tr16_b64(&Vs[g * 4 + (n >> 2)][d * 16 + (n & 3) * 4]);
-          acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pbs, acc[d], 0, 0, 0);
-          acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pls, acc[d], 0, 0, 0);
+          for (int d = 0; d < 8; ++d) {
+            // A = V^T fragment: lane (dim = d*16 + n, g) <- tokens g*4 + 0..3 (transpose read)
+            const shortx4 vf = lds_read_tr16_b64(&Vs[g * 4 + (n >> 2)][d * 16 + (n & 3) * 4]);
+            acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pbs, acc[d], 0, 0, 0);
+            acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pls, acc[d], 0, 0, 0);
+          }
+        } else {
+          Pack16 ph, pl;
+          ph.u = make_uint4(hi[0][0], hi[0][1], hi[1][0], hi[1][1]);
+          pl.u = make_uint4(lo[0][0], lo[0][1], lo[1][0], lo[1][1]);
+#pragma unroll
+          for (int d = 0; d < 8; ++d) {
+            // A = V^T fragment of both tiles: summation labels g*8 + 0..3 <- tokens g*4 + 0..3 of tile 0,
+            // labels g*8 + 4..7 <- the same tokens of tile 1
+            const shortx4 v0 = lds_read_tr16_b64(&Vs[g * 4 + (n >> 2)][d * 16 + (n & 3) * 4]);
+            const shortx4 v1 = lds_read_tr16_b64(&Vs[kTile + g * 4 + (n >> 2)][d * 16 + (n & 3) * 4]);
+            Pack16 vf;
+            vf.u = make_uint4(__builtin_bit_cast(uint2, v0).x, __builtin_bit_cast(uint2, v0).y,
+                              __builtin_bit_cast(uint2, v1).x, __builtin_bit_cast(uint2, v1).y);
+            acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, ph.v, acc[d], 0, 0, 0);
+            acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pl.v, acc[d], 0, 0, 0);
+          }
         }
       }
     }
@@ -340,7 +442,7 @@ void paged_decode_kernel(const DecodeParams p) {
           uint2 st;
           st.x = pack_bf16x2(acc[d][0] * inv, acc[d][1] * inv);
           st.y = pack_bf16x2(acc[d][2] * inv, acc[d][3] * inv);
-          *reinterpret_cast<uint2 *>(o + d * 16 + g * 4) = st;
+          *reinterpret_cast<uint2 *>(o + lds_col_dim<KV8>(d * 16 + g * 4)) = st;
         }
       }
     } else {
@@ -350,7 +452,7 @@ void paged_decode_kernel(const DecodeParams p) {
         float *po = p.part_o + (slot + head) * kDh;
 #pragma unroll
         for (int d = 0; d < 8; ++d)
-          *reinterpret_cast<float4 *>(po + d * 16 + g * 4) =
+          *reinterpret_cast<float4 *>(po + lds_col_dim<KV8>(d * 16 + g * 4)) =
               make_float4(acc[d][0] * vscale, acc[d][1] * vscale, acc[d][2] * vscale,
                           acc[d][3] * vscale);
         if (g == 0) *reinterpret_cast<float2 *>(p.part_ml + (slot + head) * 2) = make_float2(m_run, l_run);
@@ -535,8 +637,9 @@ extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void
   const dim3 g(static_cast<unsigned>(grid));
   const bool f8 = kv_dtype == TLF_KV_FP8_E4M3;
   const int pf = decode_prefetch();
+// e4m3 rows: two tiles per trip where the bf16 image of both fits LDS (up to 8 KV heads)
 #define TLF_DECODE_PF(NW, F8, PF) \
-  hipLaunchKernelGGL((paged_decode_kernel<NW, F8, PF>), g, dim3(NW * 64), 0, s, p)
+  hipLaunchKernelGGL((paged_decode_kernel<NW, F8, PF, (F8 && NW <= 8 && PF == 1 ? 2 : 1)>), g, dim3(NW * 64), 0, s, p)
 #define TLF_DECODE(NW)                                        \
   if (f8) {                                                   \
     if (pf == 1) TLF_DECODE_PF(NW, true, 1);                  \
