@@ -29,6 +29,13 @@ FLAGS = [
 ]
 
 
+# Extra flags per source file.  The attention kernels never compute with NaNs (masked scores are -inf and the
+# -inf - -inf cases are handled explicitly): without NaNs to quiet, a maximum is one instruction instead of three.
+EXTRA_FLAGS = {
+    "prefill_attn.hip": ["-fno-honor-nans"],
+}
+
+
 def sources():
     return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
 
@@ -51,7 +58,7 @@ def build(force: bool = True, verbose: bool = True) -> str:
         objs.append(obj)
         if not force and _newer(obj, [os.path.join(CSRC, src)] + headers):
             continue
-        jobs.append(["hipcc", *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj])
+        jobs.append(["hipcc", *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj])
 
     def run(cmd):
         if verbose:

@@ -16,14 +16,58 @@
 //                                       ds_read_b64_tr_b16 (LDS transpose read)
 // The rows of the K operand are permuted so that the S^T accumulator layout of
 // two 16-token sub-tiles is exactly the 32-token B operand of the second product:
-// P never leaves registers.  P is fed as a bf16 hi + lo pair.
+// P never leaves registers.
+//
+// The second product runs in fp16 (v_mfma_f32_16x16x32_f16): P lies in [0, 1], where fp16 keeps 11
+// significant bits (a single bf16 P, 8 bits, misses the 1e-3 relative-L2 bar against an exact softmax; a
+// bf16 hi + lo pair meets it at twice the MFMAs and three more vector-ALU operations per score), and V is
+// converted to fp16 once, when its tile is staged: exact for e4m3 rows, exact for bf16 rows between 6.1e-5
+// and 65504 in magnitude (smaller values keep 2^-24 absolute resolution, larger ones saturate at 65504:
+// the conversion rounds toward zero, which never produces an infinity).
 #include "common.h"
 
 namespace tlf {
 
 constexpr int kPDh = 128;
 constexpr int kBKV = 64;            // K/V tokens per LDS tile
-constexpr int kPRow = kPDh + 8;     // padded LDS row (elements)
+// Padded LDS rows (elements; LDS has 32 banks of 4 bytes).  K fragments are read 16 bytes per lane from 8
+// consecutive rows at a time: 272-byte rows.  V is read transposed, 8 bytes per lane, 4 lanes per row and
+// 4 rows at a time: 288-byte rows.
+constexpr int kPRowK = kPDh + 8;
+constexpr int kPRowV = kPDh + 16;
+typedef _Float16 f16x8 __attribute__((__vector_size__(8 * sizeof(_Float16))));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+
+// LDS row of token t (0..63) of a K tile: within each half of 32 tokens, token 8 a + 4 s + b sits in row
+// 16 s + 4 a + b, so that the 16 rows a fragment read addresses (tokens 8 a + b, or 8 a + 4 + b) are
+// consecutive.
+__device__ __forceinline__ int k_tile_row(int t) {
+  return (t & 32) | ((t & 4) << 2) | ((t & 24) >> 1) | (t & 3);
+}
+
+// Head dimension held by LDS column c of a K or V tile.  bf16 rows are stored as they come.  e4m3 rows are
+// stored with their 16-byte halves regrouped (columns 0..63: dims 16 j + 0..7, columns 64..127: dims
+// 16 j + 8..15) so that the conversion's LDS writes are conflict free; the first product sums over columns
+// (q is read with the same permutation) and the second product's output rows are columns (mapped back when
+// written).  Runs of 8 columns stay runs of 8 dims.
+template <bool KV8>
+__device__ __forceinline__ int tile_col_dim(int c) {
+  if (!KV8) return c;
+  const int j = (c >> 3) & 7;
+  return j * 16 + (c >= 64 ? 8 : 0) + (c & 7);
+}
+
+// Two bf16 (one dword) -> two fp16 (see the head of this file for the range).
+__device__ __forceinline__ unsigned int bf16x2_to_f16x2(unsigned int w) {
+  return __builtin_bit_cast(unsigned int,
+                            __builtin_amdgcn_cvt_pkrtz(__uint_as_float(w << 16), __uint_as_float(w & 0xffff0000u)));
+}
+__device__ __forceinline__ unsigned int pack_f16x2(float lo, float hi) {  // round to nearest even
+  f16x2 r;
+  r[0] = static_cast<_Float16>(lo);
+  r[1] = static_cast<_Float16>(hi);
+  return __builtin_bit_cast(unsigned int, r);
+}
 constexpr float kPLog2e = 1.4426950408889634f;
 
 struct PrefillParams {
@@ -59,12 +103,46 @@ __device__ __forceinline__ void fp8x16_to_bf16(const uint4 &in, uint4 &lo, uint4
   fp8x4_to_bf16x4(in.z, hi.x, hi.y);
   fp8x4_to_bf16x4(in.w, hi.z, hi.w);
 }
+__device__ __forceinline__ void fp8x4_to_f16x4(unsigned int w, unsigned int &lo, unsigned int &hi) {
+  lo = __builtin_bit_cast(unsigned int, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false));
+  hi = __builtin_bit_cast(unsigned int, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true));
+}
+__device__ __forceinline__ void fp8x16_to_f16(const uint4 &in, uint4 &lo, uint4 &hi) {
+  fp8x4_to_f16x4(in.x, lo.x, lo.y);
+  fp8x4_to_f16x4(in.y, lo.z, lo.w);
+  fp8x4_to_f16x4(in.z, hi.x, hi.y);
+  fp8x4_to_f16x4(in.w, hi.z, hi.w);
+}
+
+// acc[d0 .. d0 + 3] *= alpha unless alpha == 1 in every lane.
+__device__ __forceinline__ void rescale16(floatx4 (&acc)[8], int d0, float alpha) {
+  const unsigned long long moved = __builtin_amdgcn_ballot_w64(alpha != 1.0f);
+  float t[16];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) t[e] = acc[d0 + e / 4][e % 4];
+  asm volatile(
+      "s_cmp_eq_u64 %[m], 0\n\t"
+      "s_cbranch_scc1 .Ltlf_keep%=\n\t"
+      "v_mul_f32_e32 %0, %[a], %0\n\tv_mul_f32_e32 %1, %[a], %1\n\tv_mul_f32_e32 %2, %[a], %2\n\t"
+      "v_mul_f32_e32 %3, %[a], %3\n\tv_mul_f32_e32 %4, %[a], %4\n\tv_mul_f32_e32 %5, %[a], %5\n\t"
+      "v_mul_f32_e32 %6, %[a], %6\n\tv_mul_f32_e32 %7, %[a], %7\n\tv_mul_f32_e32 %8, %[a], %8\n\t"
+      "v_mul_f32_e32 %9, %[a], %9\n\tv_mul_f32_e32 %10, %[a], %10\n\tv_mul_f32_e32 %11, %[a], %11\n\t"
+      "v_mul_f32_e32 %12, %[a], %12\n\tv_mul_f32_e32 %13, %[a], %13\n\tv_mul_f32_e32 %14, %[a], %14\n\t"
+      "v_mul_f32_e32 %15, %[a], %15\n"
+      ".Ltlf_keep%=:"
+      : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]), "+v"(t[7]),
+        "+v"(t[8]), "+v"(t[9]), "+v"(t[10]), "+v"(t[11]), "+v"(t[12]), "+v"(t[13]), "+v"(t[14]), "+v"(t[15])
+      : [a] "v"(alpha), [m] "s"(moved)
+      : "scc");
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[d0 + e / 4][e % 4] = t[e];
+}
 
 template <int CT, bool KV8>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))  // 256 registers: two workgroups per CU
 void prefill_attn_kernel(const PrefillParams p) {
-  __shared__ __attribute__((aligned(16))) unsigned short Ks[kBKV][kPRow];
-  __shared__ __attribute__((aligned(16))) unsigned short Vs[kBKV][kPRow];
+  __shared__ __attribute__((aligned(16))) unsigned short Ks[kBKV][kPRowK];  // bf16, rows in k_tile_row order
+  __shared__ __attribute__((aligned(16))) unsigned short Vs[kBKV][kPRowV];  // fp16
   const int seq = blockIdx.z;
   const int h = blockIdx.y;
   const int group = p.num_q_heads / p.num_kv_heads;
@@ -96,7 +174,7 @@ void prefill_attn_kernel(const PrefillParams p) {
     for (int kc = 0; kc < 4; ++kc) {
       Pack16 t;
       t.u = make_uint4(0, 0, 0, 0);
-      if (uok[c]) t.u = *reinterpret_cast<const uint4 *>(qp + kc * 32 + g * 8);
+      if (uok[c]) t.u = *reinterpret_cast<const uint4 *>(qp + tile_col_dim<KV8>(kc * 32 + g * 8));
       qf[c][kc] = t.v;
     }
   }
@@ -159,17 +237,21 @@ void prefill_attn_kernel(const PrefillParams p) {
 #pragma unroll
     for (int i = 0; i < kPasses; ++i) {
       const int t = i * kRowsPerPass + trow;
+      const int kr = k_tile_row(t);
       if (KV8) {
+        // a thread holds dims 16 ch .. 16 ch + 15: columns 8 ch .. and 64 + 8 ch .. (tile_col_dim)
         uint4 lo, hi;
         fp8x16_to_bf16(kreg[i], lo, hi);
-        *reinterpret_cast<uint4 *>(&Ks[t][ch * 16]) = lo;
-        *reinterpret_cast<uint4 *>(&Ks[t][ch * 16 + 8]) = hi;
-        fp8x16_to_bf16(vreg[i], lo, hi);
-        *reinterpret_cast<uint4 *>(&Vs[t][ch * 16]) = lo;
-        *reinterpret_cast<uint4 *>(&Vs[t][ch * 16 + 8]) = hi;
+        *reinterpret_cast<uint4 *>(&Ks[kr][ch * 8]) = lo;
+        *reinterpret_cast<uint4 *>(&Ks[kr][64 + ch * 8]) = hi;
+        fp8x16_to_f16(vreg[i], lo, hi);
+        *reinterpret_cast<uint4 *>(&Vs[t][ch * 8]) = lo;
+        *reinterpret_cast<uint4 *>(&Vs[t][64 + ch * 8]) = hi;
       } else {
-        *reinterpret_cast<uint4 *>(&Ks[t][ch * 8]) = kreg[i];
-        *reinterpret_cast<uint4 *>(&Vs[t][ch * 8]) = vreg[i];
+        *reinterpret_cast<uint4 *>(&Ks[kr][ch * 8]) = kreg[i];
+        *reinterpret_cast<uint4 *>(&Vs[t][ch * 8]) =
+            make_uint4(bf16x2_to_f16x2(vreg[i].x), bf16x2_to_f16x2(vreg[i].y), bf16x2_to_f16x2(vreg[i].z),
+                       bf16x2_to_f16x2(vreg[i].w));
       }
     }
   };
@@ -202,12 +284,12 @@ void prefill_attn_kernel(const PrefillParams p) {
         s0[c] = floatx4{0.f, 0.f, 0.f, 0.f};
         s1[c] = floatx4{0.f, 0.f, 0.f, 0.f};
       }
-      const int tr0 = hh * 32 + (n >> 2) * 8 + (n & 3);
+      const int tr0 = hh * 32 + n;  // k_tile_row of token hh*32 + (n/4)*8 + n%4; the token 4 further on is 16 rows on
 #pragma unroll
       for (int kc = 0; kc < 4; ++kc) {
         Pack16 a0, a1;
         a0.u = *reinterpret_cast<const uint4 *>(&Ks[tr0][kc * 32 + g * 8]);
-        a1.u = *reinterpret_cast<const uint4 *>(&Ks[tr0 + 4][kc * 32 + g * 8]);
+        a1.u = *reinterpret_cast<const uint4 *>(&Ks[tr0 + 16][kc * 32 + g * 8]);
 #pragma unroll
         for (int c = 0; c < CT; ++c) {
           s0[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0.v, qf[c][kc], s0[c], 0, 0, 0);
@@ -215,13 +297,13 @@ void prefill_attn_kernel(const PrefillParams p) {
         }
       }
       // lane (n, g) of column tile c holds tokens kv0 + hh*32 + g*8 + j, j = 0..7
-      bf16x8 ph[CT], pl[CT];
+      f16x8 ph[CT];
 #pragma unroll
       for (int c = 0; c < CT; ++c) {
         // (the softmax is where this kernel's vector-ALU time goes: raw v_exp_f32, one fused
-        // multiply-add per score, no mask arithmetic on tiles that lie wholly below the diagonal)
+        // multiply-add per score, no mask arithmetic on tiles that lie wholly below the diagonal,
+        // P converted two scores per instruction)
         float sv[8];
-        float mt = -INFINITY;
         if (need_mask) {  // workgroup-uniform
           const int tbase = kv0 + hh * 32 + g * 8;
           const int limit = min(shift + urow[c], lk - 1);  // last visible key of this unit
@@ -229,38 +311,34 @@ void prefill_attn_kernel(const PrefillParams p) {
           for (int j = 0; j < 8; ++j) {
             const float raw = j < 4 ? s0[c][j] : s1[c][j - 4];
             sv[j] = tbase + j <= limit ? raw : -INFINITY;
-            mt = fmaxf(mt, sv[j]);
           }
         } else {
 #pragma unroll
-          for (int j = 0; j < 8; ++j) {
-            sv[j] = j < 4 ? s0[c][j] : s1[c][j - 4];
-            mt = fmaxf(mt, sv[j]);
-          }
+          for (int j = 0; j < 8; ++j) sv[j] = j < 4 ? s0[c][j] : s1[c][j - 4];
         }
+        float mt = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), sv[2]), fmaxf(fmaxf(sv[3], sv[4]), sv[5]));
+        mt = fmaxf(fmaxf(mt, sv[6]), sv[7]);
         mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
         mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
         // running max in the scaled (log2) domain; scale_log2 > 0, so scaling commutes with max
         const float m_new = fmaxf(m_run[c], mt * scale_log2);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
         const float alpha = __builtin_amdgcn_exp2f(m_run[c] - m_use);
-        float psum = 0.f;
+        float pv[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-          // p = 2^(s * scale - m): arguments are <= 0, a flushed denormal result is an exact 0 weight
-          const float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[j], scale_log2, -m_use));
-          psum += pv;
-          ph[c][j] = static_cast<__bf16>(pv);
-          pl[c][j] = static_cast<__bf16>(pv - static_cast<float>(ph[c][j]));
-        }
+        for (int j = 0; j < 8; ++j)  // p = 2^(s * scale - m): arguments are <= 0, a flushed denormal result is an exact 0 weight
+          pv[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[j], scale_log2, -m_use));
+        const float psum = ((pv[0] + pv[1]) + (pv[2] + pv[3])) + ((pv[4] + pv[5]) + (pv[6] + pv[7]));
+        ph[c] = __builtin_bit_cast(f16x8, make_uint4(pack_f16x2(pv[0], pv[1]), pack_f16x2(pv[2], pv[3]),
+                                                     pack_f16x2(pv[4], pv[5]), pack_f16x2(pv[6], pv[7])));
         l_run[c] = l_run[c] * alpha + psum;
         m_run[c] = m_new;
-        if (__any(alpha != 1.0f)) {  // wave-uniform: the running max rarely moves after the first tiles
-#pragma unroll
-          for (int d = 0; d < 8; ++d)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[c][d][i] *= alpha;
-        }
+        // Rescale of the accumulators, skipped (wave-uniform branch) while no lane's running max moved, which is
+        // the rule after the first tiles.  Branch and multiplies are one asm block per 16 accumulators, so that
+        // each accumulator stays in its register: written as a C++ branch, the scaled values land in new
+        // registers and the path that skips the rescale copies all 32 accumulators there on every tile.
+        rescale16(acc[c], 0, alpha);
+        rescale16(acc[c], 4, alpha);
       }
       // O^T += V^T . P^T ; V^T fragment: lane (dim = d*16 + n, g) <- tokens hh*32 + g*8 + 0..7
       const int vt = hh * 32 + g * 8 + (n >> 2);
@@ -268,14 +346,11 @@ void prefill_attn_kernel(const PrefillParams p) {
       for (int d = 0; d < 8; ++d) {
         const shortx4 v0 = lds_read_tr16(&Vs[vt][d * 16 + (n & 3) * 4]);
         const shortx4 v1 = lds_read_tr16(&Vs[vt + 4][d * 16 + (n & 3) * 4]);
-        Pack16 vf;
-        vf.u = make_uint4(__builtin_bit_cast(uint2, v0).x, __builtin_bit_cast(uint2, v0).y,
-                          __builtin_bit_cast(uint2, v1).x, __builtin_bit_cast(uint2, v1).y);
+        const f16x8 vf = __builtin_bit_cast(
+            f16x8, make_uint4(__builtin_bit_cast(uint2, v0).x, __builtin_bit_cast(uint2, v0).y,
+                              __builtin_bit_cast(uint2, v1).x, __builtin_bit_cast(uint2, v1).y));
 #pragma unroll
-        for (int c = 0; c < CT; ++c) {
-          acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, ph[c], acc[c][d], 0, 0, 0);
-          acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pl[c], acc[c][d], 0, 0, 0);
-        }
+        for (int c = 0; c < CT; ++c) acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, ph[c], acc[c][d], 0, 0, 0);
       }
     }
     lds_barrier();
@@ -301,7 +376,7 @@ void prefill_attn_kernel(const PrefillParams p) {
       uint2 st;
       st.x = pack_bf16x2(acc[c][d][0] * inv, acc[c][d][1] * inv);
       st.y = pack_bf16x2(acc[c][d][2] * inv, acc[c][d][3] * inv);
-      *reinterpret_cast<uint2 *>(o + d * 16 + g * 4) = st;
+      *reinterpret_cast<uint2 *>(o + tile_col_dim<KV8>(d * 16 + g * 4)) = st;
     }
   }
 }
