@@ -33,6 +33,7 @@ FLAGS = [
 # -inf - -inf cases are handled explicitly): without NaNs to quiet, a maximum is one instruction instead of three.
 EXTRA_FLAGS = {
     "prefill_attn.hip": ["-fno-honor-nans"],
+    "decode_attn.hip": ["-fno-honor-nans"],
 }
 
 

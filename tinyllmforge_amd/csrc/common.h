@@ -91,6 +91,22 @@ __device__ __forceinline__ float wave_sum(float v) {
   return v;
 }
 
+// Exchanges among the four lanes l, l ^ 16, l ^ 32, l ^ 48 on the vector ALU (v_permlane16_swap /
+// v_permlane32_swap), without the LDS round trip of a ds_bpermute: a = {row 0, row 0, row 2, row 2},
+// b = {row 1, row 1, row 3, row 3} of 16-lane rows after the first swap, lower and upper half after the second.
+__device__ __forceinline__ float max_lanes_16_32_48(float v) {
+  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+  r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float sum_lanes_16_32_48(float v) {
+  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+  r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // Orders this wave's LDS writes before its later LDS reads (other lanes' data).
 // LDS operations of one wave execute in program order; this only stops the
 // compiler from moving them across.

@@ -360,8 +360,7 @@ void paged_decode_kernel(const DecodeParams p) {
             sv[h][i] = valid ? s[h][i] * scale_log2 : -INFINITY;
             mt = fmaxf(mt, sv[h][i]);
           }
-        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        mt = max_lanes_16_32_48(mt);
         const float m_new = fmaxf(m_run, mt);
         // -inf only while every token so far sat in a skipped block: keep the exponents finite
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
@@ -426,8 +425,7 @@ void paged_decode_kernel(const DecodeParams p) {
         }
       }
     }
-    l_run += __shfl_xor(l_run, 16, 64);
-    l_run += __shfl_xor(l_run, 32, 64);
+    l_run = sum_lanes_16_32_48(l_run);
 
     // ---- finish the segment.  lane (n, g) holds O^T[dims d*16 + g*4 + i][head n]
     const int w_first = seq_first / tpw;

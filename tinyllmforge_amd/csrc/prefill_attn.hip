@@ -318,8 +318,7 @@ void prefill_attn_kernel(const PrefillParams p) {
         }
         float mt = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), sv[2]), fmaxf(fmaxf(sv[3], sv[4]), sv[5]));
         mt = fmaxf(fmaxf(mt, sv[6]), sv[7]);
-        mt = fmaxf(mt, __shfl_xor(mt, 16, 64));
-        mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
+        mt = max_lanes_16_32_48(mt);
         // running max in the scaled (log2) domain; scale_log2 > 0, so scaling commutes with max
         const float m_new = fmaxf(m_run[c], mt * scale_log2);
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
@@ -364,8 +363,7 @@ void prefill_attn_kernel(const PrefillParams p) {
 #pragma unroll
   for (int c = 0; c < CT; ++c) {
     float l = l_run[c];
-    l += __shfl_xor(l, 16, 64);
-    l += __shfl_xor(l, 32, 64);
+    l = sum_lanes_16_32_48(l);
     if (!uok[c]) continue;
     const int u = wave * CT * 16 + c * 16 + n;
     const int head = h * group + u % group;
