@@ -143,11 +143,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))  //
 void prefill_attn_kernel(const PrefillParams p) {
   __shared__ __attribute__((aligned(16))) unsigned short Ks[kBKV][kPRowK];  // bf16, rows in k_tile_row order
   __shared__ __attribute__((aligned(16))) unsigned short Vs[kBKV][kPRowV];  // fp16
-  const int seq = blockIdx.z;
-  const int h = blockIdx.y;
+  // Workgroup -> (sequence, KV head, row tile).  Workgroups go to the 8 XCDs round robin by their linear id, and
+  // each XCD has its own L2: when the (sequence, KV head) pairs divide evenly, pair j runs entirely on XCD j % 8,
+  // so the K/V rows its row tiles share are fetched into one L2 instead of eight.  Within a pair the last row
+  // tiles (the longest key ranges) are dispatched first, so that the launch ends on short workgroups.
+  int seq = blockIdx.z, h = blockIdx.y, xt = blockIdx.x;
+  const int pairs = gridDim.y * gridDim.z;
+  if (pairs % 8 == 0) {
+    const int lin = blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z);
+    const int slot = lin >> 3;
+    const int pair = (lin & 7) + 8 * (slot / static_cast<int>(gridDim.x));
+    xt = slot % static_cast<int>(gridDim.x);
+    h = pair % static_cast<int>(gridDim.y);
+    seq = pair / static_cast<int>(gridDim.y);
+  }
   const int group = p.num_q_heads / p.num_kv_heads;
   const int bq = (64 * CT) / group;  // query rows per workgroup
-  const int row0 = blockIdx.x * bq;
+  const int row0 = (gridDim.x - 1 - xt) * bq;
   const int q_begin = p.cu_q[seq];
   const int lq = p.cu_q[seq + 1] - q_begin;
   if (row0 >= lq) return;
