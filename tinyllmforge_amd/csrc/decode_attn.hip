@@ -110,16 +110,13 @@ struct TileRegs {
   bool ok;  // the tile's block-table entry names a real cache block
 };
 
-// PF = tiles in flight per wave (register prefetch depth).  PF == 1 fits 128 VGPRs, i.e. two
-// 8-wave workgroups per CU; deeper prefetch runs one workgroup per CU with up to 256 VGPRs.
-//
 // TS = 16-token tiles per loop trip.  bf16 rows: 1.  e4m3 rows: 2, so that a trip moves the same bytes per wave
 // as a bf16 trip does (a wave with 4 KB in flight per trip does not cover the latency of its own loads), and
 // the 32 tokens share one softmax step (one pair of cross-lane exchanges, one rescale) and feed the second
 // product through v_mfma_f32_16x16x32_bf16: the K index inside an MFMA is only a summation label, so label
 // g*8 + j stands for token g*4 + j%4 of tile j/4, which is where the first product left the scores.
-template <int NW, bool KV8, int PF, int TS>
-__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(PF == 1 && TS == 1 ? 4 : 2, 4)))
+template <int NW, bool KV8, int TS>
+__global__ __launch_bounds__(NW * 64) __attribute__((amdgpu_waves_per_eu(2, 4)))  // one workgroup of 8 waves per CU
 void paged_decode_kernel(const DecodeParams p) {
   constexpr int kThreads = NW * 64;
   constexpr int kTrip = TS * kTile;  // tokens per loop trip
@@ -127,6 +124,7 @@ void paged_decode_kernel(const DecodeParams p) {
   __shared__ __attribute__((aligned(16))) unsigned short lds_k[NW][kTrip][kLdsRowK];
   __shared__ __attribute__((aligned(16))) unsigned short lds_v[NW][kTrip][kLdsRowV];
   __shared__ int s_prefix[kMaxBatch + 1];  // tiles before sequence b
+  __shared__ int s_ctx[kMaxBatch];         // context length of sequence b (clamped to the table)
   __shared__ int s_wave_tot[16];
   __shared__ int s_start_b;
 
@@ -148,6 +146,7 @@ void paged_decode_kernel(const DecodeParams p) {
     int tiles = 0;
     if (b < p.batch) {
       const int c = min(p.context_lens[b], max_ctx);
+      s_ctx[b] = c;
       tiles = c > 0 ? (c + kTile - 1) / kTile : 0;
     }
     int incl = tiles;
@@ -198,101 +197,134 @@ void paged_decode_kernel(const DecodeParams p) {
   const float vscale = KV8 ? p.v_scale[w] : 1.0f;
   const float scale_log2 = p.scale_log2 * kscale;
 
-  int b = s_start_b;
-  int cur = ts;
-  while (cur < te) {
-    while (s_prefix[b + 1] <= cur) ++b;  // skip empty sequences (uniform)
-    const int seq_first = s_prefix[b];
-    const int seq_end = s_prefix[b + 1];
-    const int seg_end = min(te, seq_end);
-    const int ctx = min(p.context_lens[b], max_ctx);
-    const int t_begin = (cur - seq_first) * kTile;
-    const int t_end = min(ctx, (seg_end - seq_first) * kTile);
-
-    // Q as the B operand of S^T = K . Q^T: lane (n, g) holds q[head n][c*32 + g*8 .. +8].
+  // A segment = the part of one sequence that lies in this workgroup's share: sequence b, whose tiles are
+  // [seq_first, seq_end) of the flat list, tokens [t_begin, t_end); last = nothing of the share lies behind it.
+  // (plain scalars, all wave-uniform)
+#define TLF_SEG_DECL(P) int P##b, P##seq_first, P##seq_end, P##t_begin, P##t_end, P##last
+#define TLF_SEG_MAKE(P, CUR, B0)                                          \
+  {                                                                        \
+    int b_ = (B0);                                                         \
+    while (s_prefix[b_ + 1] <= (CUR)) ++b_; /* skip empty sequences */     \
+    P##b = b_;                                                             \
+    P##seq_first = s_prefix[b_];                                           \
+    P##seq_end = s_prefix[b_ + 1];                                         \
+    const int seg_end_ = min(te, P##seq_end);                              \
+    P##t_begin = ((CUR) - P##seq_first) * kTile;                           \
+    P##t_end = min(s_ctx[b_], (seg_end_ - P##seq_first) * kTile);          \
+    P##last = seg_end_ >= te;                                              \
+  }
+  // What a segment needs before its first tile: q as the B operand of S^T = K . Q^T (lane (n, g) holds
+  // q[head n][c*32 + g*8 .. +8]) and its block-table entries.  Lane i holds entry bt_base + i (64 blocks at a
+  // time), and a tile's entry is read out of that register by lane index: a per-tile fetch would sit in the
+  // in-order load queue between the tile loads, and waiting for it would drain the tile loads issued before it.
+  struct SegRegs {
     bf16x8 qf[4];
-    {
-      const unsigned short *qp = p.q + b * p.q_stride + static_cast<int64_t>(head) * kDh;
+    int bt_vec, bt_base;
+  };
+  auto fetch_seg = [&](int sb, int t_begin, SegRegs &r) {
+    const unsigned short *qp = p.q + sb * p.q_stride + static_cast<int64_t>(head) * kDh;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        Pack16 t;
-        t.u = make_uint4(0, 0, 0, 0);
-        if (head_ok) t.u = *reinterpret_cast<const uint4 *>(qp + lds_col_dim<KV8>(c * 32 + g * 8));
-        qf[c] = t.v;
-      }
+    for (int c = 0; c < 4; ++c) {
+      Pack16 t;
+      t.u = make_uint4(0, 0, 0, 0);
+      if (head_ok) t.u = *reinterpret_cast<const uint4 *>(qp + lds_col_dim<KV8>(c * 32 + g * 8));
+      r.qf[c] = t.v;
     }
-    // Block-table entries: lane i holds entry bt_base + i (64 blocks at a time), and a tile's entry is read out of
-    // that register by lane index.  A per-tile fetch would sit in the in-order load queue between the tile loads,
-    // and waiting for it would drain the tile loads issued before it.
-    const int32_t *bt = p.block_tables + b * p.bt_stride;
-    int bt_base = t_begin / p.block_size;
-    int bt_vec = bt[min(bt_base + lane, p.max_blocks - 1)];
-    auto block_of = [&](int tok) {  // tok is wave-uniform and not before the tokens asked for earlier
-      const int bi = __builtin_amdgcn_readfirstlane(tok / p.block_size);
-      if (bi - bt_base >= 64) {  // uniform, once per 64 blocks
-        bt_base = bi;
-        bt_vec = bt[min(bt_base + lane, p.max_blocks - 1)];
-      }
-      return __builtin_amdgcn_readlane(bt_vec, bi - bt_base);
-    };
+    r.bt_base = t_begin / p.block_size;
+    r.bt_vec = (p.block_tables + sb * p.bt_stride)[min(r.bt_base + lane, p.max_blocks - 1)];
+  };
 
-    // Issue the loads of the tile starting at token t0 (a tile never straddles a block); blk is its
-    // block-table entry.  The address is a wave-uniform base (the tile's first row) plus a per-lane byte
-    // offset that never changes: no vector-ALU address arithmetic per tile.  A tile that lies wholly inside
-    // the segment (all but a segment's last) loads without predicates.
-    // bf16: 4 tokens x 16 chunks of 8 elements per instruction; e4m3: 8 tokens x 8 chunks of 16
-    const unsigned int lane_off = KV8 ? static_cast<unsigned int>((lane >> 3) * row_elems + w * kDh + (lane & 7) * 16)
-                                      : static_cast<unsigned int>((g * row_elems + w * kDh + n * 8) * 2);
-    const unsigned int load_stride = static_cast<unsigned int>(KV8 ? 8 * row_elems : 4 * row_elems * 2);
-    auto load_tile = [&](int t0, int blk, TileRegs<KV8> &r) {
-      const int bi = t0 / p.block_size;
-      const bool ok = blk >= 0 && blk < p.num_cache_blocks;
-      const int64_t tok0 = static_cast<int64_t>(ok ? blk : 0) * p.block_size + (t0 - bi * p.block_size);
-      const int64_t base = tok0 * row_elems * (KV8 ? 1 : 2);
-      const unsigned char *kb = p.k_cache + base, *vb = p.v_cache + base;
-      r.ok = ok;
-      if (ok && t0 + kTile <= t_end) {  // uniform
+  // Issue the loads of the tile starting at token t0 (a tile never straddles a block); blk is its
+  // block-table entry.  The address is a wave-uniform base (the tile's first row) plus a per-lane byte
+  // offset that never changes: no vector-ALU address arithmetic per tile.  A tile that lies wholly inside
+  // the segment (all but a segment's last) loads without predicates.
+  // bf16: 4 tokens x 16 chunks of 8 elements per instruction; e4m3: 8 tokens x 8 chunks of 16
+  const unsigned int lane_off = KV8 ? static_cast<unsigned int>((lane >> 3) * row_elems + w * kDh + (lane & 7) * 16)
+                                    : static_cast<unsigned int>((g * row_elems + w * kDh + n * 8) * 2);
+  const unsigned int load_stride = static_cast<unsigned int>(KV8 ? 8 * row_elems : 4 * row_elems * 2);
+  auto load_tile = [&](int t0, int t_end, int blk, TileRegs<KV8> &r) {
+    const int bi = t0 / p.block_size;
+    const bool ok = blk >= 0 && blk < p.num_cache_blocks;
+    const int64_t tok0 = static_cast<int64_t>(ok ? blk : 0) * p.block_size + (t0 - bi * p.block_size);
+    const int64_t base = tok0 * row_elems * (KV8 ? 1 : 2);
+    const unsigned char *kb = p.k_cache + base, *vb = p.v_cache + base;
+    r.ok = ok;
+    if (ok && t0 + kTile <= t_end) {  // uniform
 #pragma unroll
-        for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
+      for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
+        r.k[i] = load_nt_u4(kb + (lane_off + i * load_stride));
+        r.v[i] = load_nt_u4(vb + (lane_off + i * load_stride));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
+        const int tt = KV8 ? i * 8 + (lane >> 3) : i * 4 + g;
+        r.k[i] = make_uint4(0, 0, 0, 0);
+        r.v[i] = make_uint4(0, 0, 0, 0);
+        if (ok && (t0 + tt) < t_end) {
           r.k[i] = load_nt_u4(kb + (lane_off + i * load_stride));
           r.v[i] = load_nt_u4(vb + (lane_off + i * load_stride));
         }
+      }
+    }
+  };
+  // the tiles of the trip that starts at token t0 of a segment that ends at t_end, block-table entries from
+  // (bt_vec, bt_base); a tile at or past t_end is not loaded
+  TileRegs<KV8> regs[TS];
+  auto load_trip = [&](int t0, int t_end, int bt_vec, int bt_base) {
+#pragma unroll
+    for (int h = 0; h < TS; ++h) {
+      const int tj = t0 + h * kTile;
+      if (tj < t_end) {
+        const int bi = __builtin_amdgcn_readfirstlane(tj / p.block_size);
+        load_tile(tj, t_end, __builtin_amdgcn_readlane(bt_vec, bi - bt_base), regs[h]);
+      }
+    }
+  };
+  auto store_tile = [&](const TileRegs<KV8> &r, int row0) {
+    unsigned short(*Ks)[kLdsRowK] = lds_k[w] + row0;
+    unsigned short(*Vs)[kLdsRowV] = lds_v[w] + row0;
+#pragma unroll
+    for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
+      if (KV8) {
+        // a lane holds dims 16 c .. 16 c + 15 (c = lane % 8): the first eight go to LDS columns 8 c ..,
+        // the other eight to columns 64 + 8 c .., so that 8 lanes write 128 contiguous bytes (lds_col_dim)
+        const int tt = i * 8 + (lane >> 3);
+        const int ch = (lane & 7) * 8;
+        uint4 lo, hi;
+        fp8x16_to_bf16x16(r.k[i], lo, hi);
+        *reinterpret_cast<uint4 *>(&Ks[tt][ch]) = lo;
+        *reinterpret_cast<uint4 *>(&Ks[tt][64 + ch]) = hi;
+        fp8x16_to_bf16x16(r.v[i], lo, hi);
+        *reinterpret_cast<uint4 *>(&Vs[tt][ch]) = lo;
+        *reinterpret_cast<uint4 *>(&Vs[tt][64 + ch]) = hi;
       } else {
-#pragma unroll
-        for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
-          const int tt = KV8 ? i * 8 + (lane >> 3) : i * 4 + g;
-          r.k[i] = make_uint4(0, 0, 0, 0);
-          r.v[i] = make_uint4(0, 0, 0, 0);
-          if (ok && (t0 + tt) < t_end) {
-            r.k[i] = load_nt_u4(kb + (lane_off + i * load_stride));
-            r.v[i] = load_nt_u4(vb + (lane_off + i * load_stride));
-          }
-        }
+        *reinterpret_cast<uint4 *>(&Ks[i * 4 + g][n * 8]) = r.k[i];
+        *reinterpret_cast<uint4 *>(&Vs[i * 4 + g][n * 8]) = r.v[i];
       }
-    };
-    auto store_tile = [&](const TileRegs<KV8> &r, int row0) {
-      unsigned short(*Ks)[kLdsRowK] = lds_k[w] + row0;
-      unsigned short(*Vs)[kLdsRowV] = lds_v[w] + row0;
-#pragma unroll
-      for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
-        if (KV8) {
-          // a lane holds dims 16 c .. 16 c + 15 (c = lane % 8): the first eight go to LDS columns 8 c ..,
-          // the other eight to columns 64 + 8 c .., so that 8 lanes write 128 contiguous bytes (lds_col_dim)
-          const int tt = i * 8 + (lane >> 3);
-          const int ch = (lane & 7) * 8;
-          uint4 lo, hi;
-          fp8x16_to_bf16x16(r.k[i], lo, hi);
-          *reinterpret_cast<uint4 *>(&Ks[tt][ch]) = lo;
-          *reinterpret_cast<uint4 *>(&Ks[tt][64 + ch]) = hi;
-          fp8x16_to_bf16x16(r.v[i], lo, hi);
-          *reinterpret_cast<uint4 *>(&Vs[tt][ch]) = lo;
-          *reinterpret_cast<uint4 *>(&Vs[tt][64 + ch]) = hi;
-        } else {
-          *reinterpret_cast<uint4 *>(&Ks[i * 4 + g][n * 8]) = r.k[i];
-          *reinterpret_cast<uint4 *>(&Vs[i * 4 + g][n * 8]) = r.v[i];
-        }
-      }
-    };
+    }
+  };
+
+
+  // One trip is in flight per wave (deeper register prefetch was measured and is no faster: the stream is not
+  // bound by this wave's latency once every CU has 64 KB in flight).  What is pipelined is the change of
+  // segment: q and the block-table entries of the next segment are fetched while the current one runs, and the
+  // first trip of the next segment is loaded during the last trip of the current one, so a workgroup whose
+  // share covers several sequences does not stop streaming between them.
+  TLF_SEG_DECL(sg_);
+  TLF_SEG_DECL(sn_);
+  TLF_SEG_MAKE(sg_, ts, s_start_b)
+  SegRegs cur_regs, next_regs;
+  fetch_seg(sg_b, sg_t_begin, next_regs);
+  load_trip(sg_t_begin, sg_t_end, next_regs.bt_vec, next_regs.bt_base);
+  while (true) {
+    cur_regs = next_regs;
+    sn_b = sg_b; sn_seq_first = sg_seq_first; sn_seq_end = sg_seq_end; sn_t_begin = 0; sn_t_end = 0; sn_last = 1;
+    if (!sg_last) {
+      TLF_SEG_MAKE(sn_, sg_seq_end, sg_b + 1)
+      fetch_seg(sn_b, sn_t_begin, next_regs);
+    }
+    const bf16x8(&qf)[4] = cur_regs.qf;
 
     floatx4 acc[8];
 #pragma unroll
@@ -300,141 +332,135 @@ void paged_decode_kernel(const DecodeParams p) {
     float m_run = -INFINITY;  // running max (log2 domain), identical in the 4 lanes of a head
     float l_run = 0.f;        // this lane's share of the running sum
 
-    // PF trips are kept in flight: tile h of trip j of a group of PF lives in regs[j][h].
-    TileRegs<KV8> regs[PF][TS];
-#pragma unroll
-    for (int j = 0; j < PF; ++j)
+    for (int t0 = sg_t_begin; t0 < sg_t_end; t0 += kTrip) {
+      wave_lds_fence();  // previous trip's LDS reads are done
+      bool tile_ok[TS];
 #pragma unroll
       for (int h = 0; h < TS; ++h) {
-        const int tj = t_begin + j * kTrip + h * kTile;
-        regs[j][h].ok = false;
-        if (tj < t_end) load_tile(tj, block_of(tj), regs[j][h]);
+        // a tile past the end of the segment (second tile of the last trip) was never loaded: zeros, masked below
+        if (t0 + h * kTile >= sg_t_end) {
+#pragma unroll
+          for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
+            regs[h].k[i] = make_uint4(0, 0, 0, 0);
+            regs[h].v[i] = make_uint4(0, 0, 0, 0);
+          }
+          regs[h].ok = false;
+        }
+        store_tile(regs[h], h * kTile);
+        tile_ok[h] = regs[h].ok;
       }
-    for (int tg = t_begin; tg < t_end; tg += PF * kTrip) {
-#pragma unroll
-      for (int j = 0; j < PF; ++j) {
-        const int t0 = tg + j * kTrip;
-        if (t0 >= t_end) break;  // uniform
-        wave_lds_fence();  // previous trip's LDS reads are done
-        bool tile_ok[TS];
-#pragma unroll
-        for (int h = 0; h < TS; ++h) {
-          // a tile past the end of the segment (second tile of the last trip) was never loaded: zeros, masked below
-          if (t0 + h * kTile >= t_end) {
-#pragma unroll
-            for (int i = 0; i < TileRegs<KV8>::kLoads; ++i) {
-              regs[j][h].k[i] = make_uint4(0, 0, 0, 0);
-              regs[j][h].v[i] = make_uint4(0, 0, 0, 0);
-            }
-            regs[j][h].ok = false;
+      wave_lds_fence();
+      {
+        // next trip: of this segment, or the first of the next one (t_end 0 when there is none: nothing loads)
+        const bool more = t0 + kTrip < sg_t_end;
+        if (more) {  // 64 block-table entries per register: move the window on (uniform, rare)
+          const int bi = __builtin_amdgcn_readfirstlane((t0 + kTrip + (TS - 1) * kTile) / p.block_size);
+          if (bi - cur_regs.bt_base >= 64) {
+            cur_regs.bt_base = (t0 + kTrip) / p.block_size;
+            cur_regs.bt_vec =
+                (p.block_tables + sg_b * p.bt_stride)[min(cur_regs.bt_base + lane, p.max_blocks - 1)];
           }
-          store_tile(regs[j][h], h * kTile);
-          tile_ok[h] = regs[j][h].ok;
         }
-        wave_lds_fence();
-#pragma unroll
-        for (int h = 0; h < TS; ++h) {
-          const int tn = t0 + PF * kTrip + h * kTile;
-          if (tn < t_end) load_tile(tn, block_of(tn), regs[j][h]);
-        }
+        load_trip(more ? t0 + kTrip : sn_t_begin, more ? sg_t_end : sn_t_end,
+                  more ? cur_regs.bt_vec : next_regs.bt_vec, more ? cur_regs.bt_base : next_regs.bt_base);
+      }
 
-        // S^T = K . Q^T : lane (n, g) gets tokens g*4 + i of head n, for each tile of the trip
-        floatx4 s[TS];
+      // S^T = K . Q^T : lane (n, g) gets tokens g*4 + i of head n, for each tile of the trip
+      floatx4 s[TS];
 #pragma unroll
-        for (int h = 0; h < TS; ++h) s[h] = floatx4{0.f, 0.f, 0.f, 0.f};
+      for (int h = 0; h < TS; ++h) s[h] = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int c = 0; c < 4; ++c)
-#pragma unroll
-          for (int h = 0; h < TS; ++h) {
-            Pack16 a;
-            a.u = *reinterpret_cast<const uint4 *>(&Ks[h * kTile + n][c * 32 + g * 8]);
-            s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[c], s[h], 0, 0, 0);
-          }
-        float sv[TS][4];
-        float mt = -INFINITY;
-#pragma unroll
-        for (int h = 0; h < TS; ++h)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            const bool valid = tile_ok[h] && (t0 + h * kTile + g * 4 + i) < t_end;
-            sv[h][i] = valid ? s[h][i] * scale_log2 : -INFINITY;
-            mt = fmaxf(mt, sv[h][i]);
-          }
-        mt = max_lanes_16_32_48(mt);
-        const float m_new = fmaxf(m_run, mt);
-        // -inf only while every token so far sat in a skipped block: keep the exponents finite
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        // raw v_exp_f32: results below 2^-126 (which the library routine would denormalise) weigh nothing here
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
-        float pv[TS][4];
-        float psum = 0.f;
+      for (int c = 0; c < 4; ++c)
 #pragma unroll
         for (int h = 0; h < TS; ++h) {
-#pragma unroll
-          for (int i = 0; i < 4; ++i) pv[h][i] = __builtin_amdgcn_exp2f(sv[h][i] - m_use);
-          psum += (pv[h][0] + pv[h][1]) + (pv[h][2] + pv[h][3]);
+          Pack16 a;
+          a.u = *reinterpret_cast<const uint4 *>(&Ks[h * kTile + n][c * 32 + g * 8]);
+          s[h] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, qf[c], s[h], 0, 0, 0);
         }
-        l_run = l_run * alpha + psum;
-        m_run = m_new;
-        // P as a bf16 hi + lo pair, converted two at a time
-        unsigned int hi[TS][2], lo[TS][2];
+      float sv[TS][4];
+      float mt = -INFINITY;
 #pragma unroll
-        for (int h = 0; h < TS; ++h)
+      for (int h = 0; h < TS; ++h)
 #pragma unroll
-          for (int e = 0; e < 2; ++e) {
-            hi[h][e] = pack_bf16x2(pv[h][2 * e], pv[h][2 * e + 1]);
-            lo[h][e] = pack_bf16x2(pv[h][2 * e] - __uint_as_float(hi[h][e] << 16),
-                                   pv[h][2 * e + 1] - __uint_as_float(hi[h][e] & 0xffff0000u));
-          }
-        // the running max rarely moves after the first tiles: skip the 32 multiplies then.  The branch is
-        // wave-uniform and must stay a branch (the empty asm keeps the compiler from turning it into 32
-        // multiplies and 32 selects on every trip).
-        if (__any(alpha != 1.0f)) {
-          asm volatile("" ::);
-#pragma unroll
-          for (int d = 0; d < 8; ++d)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[d][i] *= alpha;
+        for (int i = 0; i < 4; ++i) {
+          const bool valid = tile_ok[h] && (t0 + h * kTile + g * 4 + i) < sg_t_end;
+          sv[h][i] = valid ? s[h][i] * scale_log2 : -INFINITY;
+          mt = fmaxf(mt, sv[h][i]);
         }
-        if constexpr (TS == 1) {
-          const shortx4 pbs = __builtin_bit_cast(shortx4, make_uint2(hi[0][0], hi[0][1]));
-          const shortx4 pls = __builtin_bit_cast(shortx4, make_uint2(lo[0][0], lo[0][1]));
+      mt = max_lanes_16_32_48(mt);
+      const float m_new = fmaxf(m_run, mt);
+      // -inf only while every token so far sat in a skipped block: keep the exponents finite
+      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+      // raw v_exp_f32: results below 2^-126 (which the library routine would denormalise) weigh nothing here
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
+      float pv[TS][4];
+      float psum = 0.f;
 #pragma unroll
-          for (int d = 0; d < 8; ++d) {
-            // A = V^T fragment: lane (dim = d*16 + n, g) <- tokens g*4 + 0..3 (transpose read)
-            const shortx4 vf = lds_read_tr16_b64(&Vs[g * 4 + (n >> 2)][d * 16 + (n & 3) * 4]);
-            acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pbs, acc[d], 0, 0, 0);
-            acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pls, acc[d], 0, 0, 0);
-          }
-        } else {
-          Pack16 ph, pl;
-          ph.u = make_uint4(hi[0][0], hi[0][1], hi[1][0], hi[1][1]);
-          pl.u = make_uint4(lo[0][0], lo[0][1], lo[1][0], lo[1][1]);
+      for (int h = 0; h < TS; ++h) {
 #pragma unroll
-          for (int d = 0; d < 8; ++d) {
-            // A = V^T fragment of both tiles: summation labels g*8 + 0..3 <- tokens g*4 + 0..3 of tile 0,
-            // labels g*8 + 4..7 <- the same tokens of tile 1
-            const shortx4 v0 = lds_read_tr16_b64(&Vs[g * 4 + (n >> 2)][d * 16 + (n & 3) * 4]);
-            const shortx4 v1 = lds_read_tr16_b64(&Vs[kTile + g * 4 + (n >> 2)][d * 16 + (n & 3) * 4]);
-            Pack16 vf;
-            vf.u = make_uint4(__builtin_bit_cast(uint2, v0).x, __builtin_bit_cast(uint2, v0).y,
-                              __builtin_bit_cast(uint2, v1).x, __builtin_bit_cast(uint2, v1).y);
-            acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, ph.v, acc[d], 0, 0, 0);
-            acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pl.v, acc[d], 0, 0, 0);
-          }
+        for (int i = 0; i < 4; ++i) pv[h][i] = __builtin_amdgcn_exp2f(sv[h][i] - m_use);
+        psum += (pv[h][0] + pv[h][1]) + (pv[h][2] + pv[h][3]);
+      }
+      l_run = l_run * alpha + psum;
+      m_run = m_new;
+      // P as a bf16 hi + lo pair, converted two at a time
+      unsigned int hi[TS][2], lo[TS][2];
+#pragma unroll
+      for (int h = 0; h < TS; ++h)
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          hi[h][e] = pack_bf16x2(pv[h][2 * e], pv[h][2 * e + 1]);
+          lo[h][e] = pack_bf16x2(pv[h][2 * e] - __uint_as_float(hi[h][e] << 16),
+                                 pv[h][2 * e + 1] - __uint_as_float(hi[h][e] & 0xffff0000u));
+        }
+      // the running max rarely moves after the first tiles: skip the 32 multiplies then.  The branch is
+      // wave-uniform and must stay a branch (the empty asm keeps the compiler from turning it into 32
+      // multiplies and 32 selects on every trip).
+      if (__any(alpha != 1.0f)) {
+        asm volatile("" ::);
+#pragma unroll
+        for (int d = 0; d < 8; ++d)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[d][i] *= alpha;
+      }
+      if constexpr (TS == 1) {
+        const shortx4 pbs = __builtin_bit_cast(shortx4, make_uint2(hi[0][0], hi[0][1]));
+        const shortx4 pls = __builtin_bit_cast(shortx4, make_uint2(lo[0][0], lo[0][1]));
+#pragma unroll
+        for (int d = 0; d < 8; ++d) {
+          // A = V^T fragment: lane (dim = d*16 + n, g) <- tokens g*4 + 0..3 (transpose read)
+          const shortx4 vf = lds_read_tr16_b64(&Vs[g * 4 + (n >> 2)][d * 16 + (n & 3) * 4]);
+          acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pbs, acc[d], 0, 0, 0);
+          acc[d] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pls, acc[d], 0, 0, 0);
+        }
+      } else {
+        Pack16 ph, pl;
+        ph.u = make_uint4(hi[0][0], hi[0][1], hi[1][0], hi[1][1]);
+        pl.u = make_uint4(lo[0][0], lo[0][1], lo[1][0], lo[1][1]);
+#pragma unroll
+        for (int d = 0; d < 8; ++d) {
+          // A = V^T fragment of both tiles: summation labels g*8 + 0..3 <- tokens g*4 + 0..3 of tile 0,
+          // labels g*8 + 4..7 <- the same tokens of tile 1
+          const shortx4 v0 = lds_read_tr16_b64(&Vs[g * 4 + (n >> 2)][d * 16 + (n & 3) * 4]);
+          const shortx4 v1 = lds_read_tr16_b64(&Vs[kTile + g * 4 + (n >> 2)][d * 16 + (n & 3) * 4]);
+          Pack16 vf;
+          vf.u = make_uint4(__builtin_bit_cast(uint2, v0).x, __builtin_bit_cast(uint2, v0).y,
+                            __builtin_bit_cast(uint2, v1).x, __builtin_bit_cast(uint2, v1).y);
+          acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, ph.v, acc[d], 0, 0, 0);
+          acc[d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pl.v, acc[d], 0, 0, 0);
         }
       }
     }
     l_run = sum_lanes_16_32_48(l_run);
 
     // ---- finish the segment.  lane (n, g) holds O^T[dims d*16 + g*4 + i][head n]
-    const int w_first = seq_first / tpw;
-    const int w_last = (seq_end - 1) / tpw;
+    const int w_first = sg_seq_first / tpw;
+    const int w_last = (sg_seq_end - 1) / tpw;
     const int nseg = w_last - w_first + 1;
     if (nseg == 1) {
       if (head_ok) {
         const float inv = l_run > 0.f ? vscale / l_run : 0.f;
-        unsigned short *o = p.out + (static_cast<int64_t>(b) * p.num_q_heads + head) * kDh;
+        unsigned short *o = p.out + (static_cast<int64_t>(sg_b) * p.num_q_heads + head) * kDh;
 #pragma unroll
         for (int d = 0; d < 8; ++d) {
           uint2 st;
@@ -445,7 +471,7 @@ void paged_decode_kernel(const DecodeParams p) {
       }
     } else {
       // (workgroup, sequence) pairs form a staircase, so blockIdx + b is a unique slot
-      const int64_t slot = (static_cast<int64_t>(blockIdx.x) + b) * p.num_q_heads;
+      const int64_t slot = (static_cast<int64_t>(blockIdx.x) + sg_b) * p.num_q_heads;
       if (head_ok) {
         float *po = p.part_o + (slot + head) * kDh;
 #pragma unroll
@@ -456,11 +482,14 @@ void paged_decode_kernel(const DecodeParams p) {
         if (g == 0) *reinterpret_cast<float2 *>(p.part_ml + (slot + head) * 2) = make_float2(m_run, l_run);
       }
     }
-    if (tid == 0 && cur == seq_first)  // the share holding the sequence's first tile records its split
-      *reinterpret_cast<int2 *>(p.meta + 2 * b) = make_int2(w_first, nseg);
-    cur = seg_end;
-    ++b;
+    if (tid == 0 && sg_t_begin == 0)  // the share holding the sequence's first tile records its split
+      *reinterpret_cast<int2 *>(p.meta + 2 * sg_b) = make_int2(w_first, nseg);
+    if (sg_last) break;
+    sg_b = sn_b; sg_seq_first = sn_seq_first; sg_seq_end = sn_seq_end; sg_t_begin = sn_t_begin; sg_t_end = sn_t_end;
+    sg_last = sn_last;
   }
+#undef TLF_SEG_DECL
+#undef TLF_SEG_MAKE
 }
 
 // Merge the partials of the sequences that were cut by share boundaries.
@@ -528,8 +557,8 @@ inline int device_cu_count() {
 
 // Workgroups per CU of the persistent grid.  Measured on MI355X (config: B=64, ctx 512..4096):
 // 1 -> 109 us, 2 -> 116 us, 3 -> 119 us, 4 -> 125 us per call: fewer, longer shares mean fewer
-// partials and less contention.  TLF_DECODE_WGS_PER_CU overrides for tuning (2 and more need
-// TLF_DECODE_PREFETCH=1 to fit the register file).
+// partials and less contention.  TLF_DECODE_WGS_PER_CU overrides the grid size for tuning (one workgroup
+// is resident per CU: LDS, and a register budget of 256 per lane).
 inline int decode_wgs_per_cu() {
   static int v = 0;
   if (v == 0) {
@@ -537,18 +566,6 @@ inline int decode_wgs_per_cu() {
     if (const char *e = getenv("TLF_DECODE_WGS_PER_CU")) {
       const int x = atoi(e);
       if (x >= 1 && x <= 4) v = x;
-    }
-  }
-  return v;
-}
-
-inline int decode_prefetch() {
-  static int v = 0;
-  if (v == 0) {
-    v = 1;  // measured on MI355X: depth 2 and 3 are no faster (the stream is not latency bound)
-    if (const char *e = getenv("TLF_DECODE_PREFETCH")) {
-      const int x = atoi(e);
-      if (x >= 1 && x <= 3) v = x;
     }
   }
   return v;
@@ -634,20 +651,12 @@ extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 g(static_cast<unsigned>(grid));
   const bool f8 = kv_dtype == TLF_KV_FP8_E4M3;
-  const int pf = decode_prefetch();
-// e4m3 rows: two tiles per trip where the bf16 image of both fits LDS (up to 8 KV heads)
-#define TLF_DECODE_PF(NW, F8, PF) \
-  hipLaunchKernelGGL((paged_decode_kernel<NW, F8, PF, (F8 && NW <= 8 && PF == 1 ? 2 : 1)>), g, dim3(NW * 64), 0, s, p)
-#define TLF_DECODE(NW)                                        \
-  if (f8) {                                                   \
-    if (pf == 1) TLF_DECODE_PF(NW, true, 1);                  \
-    else if (pf == 2) TLF_DECODE_PF(NW, true, 2);             \
-    else TLF_DECODE_PF(NW, true, 3);                          \
-  } else {                                                    \
-    if (pf == 1) TLF_DECODE_PF(NW, false, 1);                 \
-    else if (pf == 2) TLF_DECODE_PF(NW, false, 2);            \
-    else TLF_DECODE_PF(NW, false, 3);                         \
-  }
+  // e4m3 rows: two tiles per trip where the bf16 image of both fits LDS (up to 8 KV heads)
+#define TLF_DECODE(NW)                                                                              \
+  if (f8)                                                                                           \
+    hipLaunchKernelGGL((paged_decode_kernel<NW, true, (NW <= 8 ? 2 : 1)>), g, dim3(NW * 64), 0, s, p); \
+  else                                                                                              \
+    hipLaunchKernelGGL((paged_decode_kernel<NW, false, 1>), g, dim3(NW * 64), 0, s, p)
   switch (num_kv_heads) {
     case 1: TLF_DECODE(1); break;
     case 2: TLF_DECODE(2); break;
@@ -657,7 +666,6 @@ extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void
     default: return TLF_E_UNSUPPORTED;
   }
 #undef TLF_DECODE
-#undef TLF_DECODE_PF
   int rc = launch_status();
   if (rc != TLF_OK) return rc;
   hipLaunchKernelGGL(paged_decode_merge_kernel, dim3((num_q_heads + 7) / 8, batch), dim3(256), 0, s, p);
