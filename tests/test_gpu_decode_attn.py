@@ -145,3 +145,71 @@ def test_decode_fp8_cache():
     got = P.paged_decode_attention(q.to(DEV), k8.to(DEV), v8.to(DEV), cl.to(DEV), bt.to(DEV), 0.0884,
                                    ks.to(DEV), vs.to(DEV)).cpu()
     check(got, ref)
+
+
+def _fp8_case(seed, Hq, Hkv, bs, ctxs, nblk, maxb=None, pad=-1):
+    Dh = 128
+    q, kc, vc, cl, bt = make_case(seed, len(ctxs), Hq, Hkv, bs, ctxs, nblk, maxb=maxb, pad=pad)
+    ks = torch.rand(Hkv, generator=torch.Generator().manual_seed(seed + 1)) * 0.02 + 0.01
+    vs = torch.rand(Hkv, generator=torch.Generator().manual_seed(seed + 2)) * 0.02 + 0.01
+    k8 = O.quantize_fp8(kc.view(-1, Hkv, Dh), ks).view(kc.shape)
+    v8 = O.quantize_fp8(vc.view(-1, Hkv, Dh), vs).view(vc.shape)
+    return q, k8, v8, cl, bt, ks, vs
+
+
+def _run_fp8(case, scale=0.0884):
+    from tinyllmforge_amd import ops as P
+    q, k8, v8, cl, bt, ks, vs = case
+    ref = O.paged_decode_attention(q, k8, v8, cl, bt, scale, ks, vs)
+    got = P.paged_decode_attention(q.to(DEV), k8.to(DEV), v8.to(DEV), cl.to(DEV), bt.to(DEV), scale,
+                                   ks.to(DEV), vs.to(DEV)).cpu()
+    return got, ref
+
+
+@pytest.mark.parametrize("Hq,Hkv,bs", [(64, 8, 256), (32, 8, 16), (16, 4, 256), (32, 16, 256)])
+def test_decode_fp8_trip_boundaries(Hq, Hkv, bs):
+    """e4m3 rows are walked two 16-token tiles per trip (one tile per trip with 16 KV heads): lengths around
+    every tile, trip and block boundary, odd tile counts, shares that start on an odd tile of a sequence."""
+    ctxs = [1, 15, 16, 17, 31, 32, 33, 47, 48, 49, 255, 256, 257, 271, 272, 273, 287, 288, 289, 511, 513, 1040]
+    nblk = sum((c + bs - 1) // bs for c in ctxs) + 3
+    got, ref = _run_fp8(_fp8_case(31, Hq, Hkv, bs, ctxs, nblk))
+    check(got, ref)
+
+
+def test_decode_fp8_many_short_sequences_and_unmapped_blocks():
+    """Several sequences per workgroup (the next sequence's first tiles are loaded during the last trip of the
+    current one), and block-table entries that name no block (-1, or past the pool) in either tile of a trip:
+    their tokens are skipped, as the bf16 path does."""
+    ge = torch.Generator().manual_seed(7)
+    ctxs = torch.randint(1, 100, (150,), generator=ge).tolist()
+    got, ref = _run_fp8(_fp8_case(33, 32, 8, 16, ctxs, sum((c + 15) // 16 for c in ctxs) + 2))
+    check(got, ref)
+    # Unmapped entries have no counterpart in the reference or the oracle (both would index some block): the
+    # e4m3 path must skip exactly the tokens the bf16 path skips.  With one scale for all heads the e4m3 result
+    # is c_v times the bf16 path's result on the same (exactly representable) rows with the softmax scale times c_k.
+    from tinyllmforge_amd import ops as P
+    q, k8, v8, cl, bt, _, _ = _fp8_case(35, 32, 8, 16, [200, 90, 33, 64], 40)
+    bt = bt.clone()
+    bt[0, 1] = -1       # second tile of the first trip
+    bt[0, 4] = 10 ** 6  # first tile of a later trip, past the pool
+    bt[1, 5] = -1       # last (partial) tile
+    bt[3, 0] = -1
+    ck, cv = 0.015625, 0.03125
+    ks, vs = torch.full((8,), ck), torch.full((8,), cv)
+    got8 = P.paged_decode_attention(q.to(DEV), k8.to(DEV), v8.to(DEV), cl.to(DEV), bt.to(DEV), 0.0884,
+                                    ks.to(DEV), vs.to(DEV)).float().cpu()
+    got16 = P.paged_decode_attention(q.to(DEV), k8.to(BF).to(DEV), v8.to(BF).to(DEV), cl.to(DEV), bt.to(DEV),
+                                     0.0884 * ck).float().cpu() * cv
+    assert (got8 - got16).abs().max().item() <= 2e-2
+    assert ((got8 - got16).norm() / got16.norm()).item() <= 1e-3
+
+
+def test_decode_segment_changes_inside_a_workgroup_bf16():
+    """bf16 rows, sequences much shorter than a workgroup's share: every workgroup changes sequence several
+    times, some sequences are cut by share boundaries, some lie inside one share."""
+    ge = torch.Generator().manual_seed(11)
+    ctxs = torch.randint(1, 400, (300,), generator=ge).tolist()
+    ctxs[17] = 0
+    ctxs[200] = 0
+    got, ref = run_both(make_case(37, len(ctxs), 32, 8, 16, ctxs, sum((c + 15) // 16 for c in ctxs) + 2))
+    check(got, ref)

@@ -116,3 +116,73 @@ def test_prefill_empty_sequence_in_batch_and_fp8_cache():
     got8 = P.varlen_prefill_attention(q.to(DEV), k8.to(DEV), v8.to(DEV), cq.to(DEV), ck.to(DEV), 20, scale,
                                       block_tables=bt.to(DEV), k_scale=ks.to(DEV), v_scale=vs.to(DEV))
     check(got8, ref8)
+
+
+def _sampled_rows_check(q, kc, vc, cq, ck, bt, scale, got, rows, k_scale=None, v_scale=None):
+    """Oracle on sampled query rows only: a single query at the end of its visible key range is the same
+    bottom-right aligned causal problem (CPU time stays in seconds for 8192-token sequences)."""
+    got = got.float().cpu()
+    num = den = 0.0
+    for seq, i in rows:
+        lq = int(cq[seq + 1] - cq[seq])
+        lk = int(ck[seq + 1] - ck[seq])
+        vis = lk - lq + i + 1
+        qi = q[int(cq[seq]) + i:int(cq[seq]) + i + 1]
+        ref = O.varlen_prefill_attention(qi, kc, vc, cu([1]), cu([vis]), scale, block_tables=bt[seq:seq + 1],
+                                         **({} if k_scale is None else dict(k_scale=k_scale, v_scale=v_scale))).float()
+        g_ = got[int(cq[seq]) + i:int(cq[seq]) + i + 1]
+        assert (g_ - ref).abs().max().item() <= 2e-2, (seq, i)
+        num += float((g_ - ref).pow(2).sum())
+        den += float(ref.pow(2).sum())
+    rel = (num / den) ** 0.5
+    assert rel <= 1e-3, f"rel l2 {rel}"
+    return rel
+
+
+@pytest.mark.parametrize("fp8", [False, True])
+def test_prefill_long_sequences_behind_cached_prefix(fp8):
+    """BASELINE configs[4] shape (64 query heads, 8 KV heads): an 8192-token prompt, and a 4096-token prompt
+    behind a 1024-token cached prefix, bf16 and e4m3 cache rows; sampled rows against the oracle.  The second
+    product runs in fp16 (P and V): this is the test of its tolerance at full length."""
+    from tinyllmforge_amd import ops as P
+    Hq, Hkv, bs, Dh = 64, 8, 256, 128
+    lens_q, lens_k = [8192, 4096, 300], [8192, 5120, 300]
+    nblk = sum((l + bs - 1) // bs for l in lens_k) + 2
+    q, kc, vc, cq, ck, bt = paged_case(41, Hq, Hkv, bs, lens_q, lens_k, nblk)
+    scale = Dh ** -0.5
+    kw, okw = {}, {}
+    if fp8:
+        ks = torch.rand(Hkv, generator=g(1)) * 0.02 + 0.01
+        vs = torch.rand(Hkv, generator=g(2)) * 0.02 + 0.01
+        kc = O.quantize_fp8(kc.view(-1, Hkv, Dh), ks).view(kc.shape)
+        vc = O.quantize_fp8(vc.view(-1, Hkv, Dh), vs).view(vc.shape)
+        kw = dict(k_scale=ks.to(DEV), v_scale=vs.to(DEV))
+        okw = dict(k_scale=ks, v_scale=vs)
+    got = P.varlen_prefill_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), cq.to(DEV), ck.to(DEV), max(lens_q), scale,
+                                     block_tables=bt.to(DEV), **kw)
+    rows = [(0, 0), (0, 1), (0, 63), (0, 64), (0, 4095), (0, 8000), (0, 8191), (1, 0), (1, 17), (1, 2048), (1, 4095),
+            (2, 0), (2, 299)]
+    rel = _sampled_rows_check(q, kc, vc, cq, ck, bt, scale, got, rows, **okw)
+    print(f"PREFILL_ERR long fp8={fp8}: rel l2 {rel:.2e}")
+
+
+@pytest.mark.parametrize("vmag", [1e-3, 1.0, 3e3])
+def test_prefill_fp16_second_product_over_the_range_of_v(vmag):
+    """V is converted to fp16 when its tile is staged: exact between 6.1e-5 and 65504 in magnitude.  Values of
+    the size of real activations, a thousand times smaller and three thousand times larger meet the tolerance
+    (relative L2; the absolute bound scales with the outputs)."""
+    from tinyllmforge_amd import ops as P
+    Hq, Hkv, Dh = 32, 8, 128
+    lens = [700, 130]
+    S = sum(lens)
+    ge = g(51)
+    q = torch.randn(S, Hq, Dh, generator=ge).to(BF)
+    k = torch.randn(S, Hkv, Dh, generator=ge).to(BF)
+    v = (torch.randn(S, Hkv, Dh, generator=ge) * vmag).to(BF)
+    c = cu(lens)
+    scale = Dh ** -0.5
+    ref = O.varlen_prefill_attention(q, k, v, c, c, scale).float()
+    got = P.varlen_prefill_attention(q.to(DEV), k.to(DEV), v.to(DEV), c.to(DEV), c.to(DEV), max(lens), scale).float().cpu()
+    rel = ((got - ref).norm() / ref.norm()).item()
+    assert rel <= 1e-3, f"rel l2 {rel}"
+    assert (got - ref).abs().max().item() <= 2e-2 * max(1.0, vmag)
