@@ -822,10 +822,18 @@ __global__ __launch_bounds__(256) void splitk_reduce_add_rmsnorm_kernel(const Ge
 // the same labelling.  A workgroup owns 16*TN output channels; its 8 waves split
 // K and the partial accumulators are summed through LDS, so nothing but the
 // final bf16 rows goes back to memory.
-template <int MT, int TN, bool W8>
-__global__ __launch_bounds__(512) void skinny_gemm_kernel(const GemmParams p) {
+//
+// PIPE: two batches of weight and activation loads in flight (see below); measured faster up to 8 tokens, where
+// a wave's stream is bound by the latency of its own loads (down projection, 1 token: 15.4 -> 11.4 us), slower
+// from 9 tokens on, where the activation fragments are twice the weight bytes of a K-block.
+template <int MT, int TN, bool W8, bool PIPE>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(PIPE ? 4 : 2, PIPE ? 4 : 8)))
+void skinny_gemm_kernel(const GemmParams p) {
   constexpr int kWaves = 8;
-  constexpr int kU = 4;  // K-blocks of 64 whose weight loads are in flight together
+  // K-blocks of 64 per batch of loads: as many as two batches fit in about 64 registers per lane (the kernel
+  // keeps to 128 registers, so that two workgroups share a CU)
+  constexpr int kRegsPerBlock = TN * (W8 ? 4 : 8) + MT * 8;
+  constexpr int kU = 2 * 4 * kRegsPerBlock <= 64 ? 4 : 2 * 2 * kRegsPerBlock <= 64 ? 2 : 1;
   __shared__ __attribute__((aligned(16))) float red[kWaves][TN * MT][64][4];
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
@@ -862,63 +870,143 @@ __global__ __launch_bounds__(512) void skinny_gemm_kernel(const GemmParams p) {
     xrow[m] = p.x + static_cast<int64_t>(xok[m] ? row : 0) * p.ldx_bytes;
   }
 
-  for (int kb0 = kb_begin; kb0 < kb_end; kb0 += kU) {
-    // issue the weight loads of up to kU K-blocks
-    uint4 wraw[kU][TN][W8 ? 1 : 2];
-#pragma unroll
-    for (int u = 0; u < kU; ++u) {
-      const int kb = kb0 + u;
-#pragma unroll
-      for (int t = 0; t < TN; ++t) {
-        if (W8) {
-          wraw[u][t][0] = make_uint4(0, 0, 0, 0);
-          if (kb < kb_end && wok[t]) wraw[u][t][0] = load_nt_u4(wrow[t] + static_cast<int64_t>(kb) * 2048);
-        } else {
-          wraw[u][t][0] = make_uint4(0, 0, 0, 0);
-          wraw[u][t][W8 ? 0 : 1] = make_uint4(0, 0, 0, 0);
-          if (kb < kb_end && wok[t]) {
+  if constexpr (PIPE) {
+    // Two batches of kU K-blocks are in flight: the loads of batch i + 1 (weights and activations) are issued
+    // before batch i is consumed.  Every load is unconditional (a K-block past the wave's range re-reads its
+    // last block, a row past N or M reads row 0; what they produce is never stored), so that the waits are
+    // counted and a batch is consumed while the next one is still on its way.
+    constexpr int kWL = W8 ? 1 : 2;  // 128-bit weight loads per lane, tile and K-block
+    struct Batch {
+      uint4 w[kU][TN][kWL];
+      uint4 x[kU][MT][2];
+    };
+    auto issue = [&](int kb0, Batch &bt) {
+  #pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        const int kb = min(kb0 + u, kb_end - 1);
+  #pragma unroll
+        for (int t = 0; t < TN; ++t) {
+          if (W8) {
+            bt.w[u][t][0] = load_nt_u4(wrow[t] + static_cast<int64_t>(kb) * 2048);
+          } else {
             const unsigned char *src = wrow[t] + (static_cast<int64_t>(kb) * kBK + g * 16) * 2;
-            wraw[u][t][0] = load_nt_u4(src);
-            wraw[u][t][W8 ? 0 : 1] = load_nt_u4(src + 16);
+            bt.w[u][t][0] = load_nt_u4(src);
+            bt.w[u][t][kWL - 1] = load_nt_u4(src + 16);
+          }
+        }
+  #pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          const unsigned char *src = xrow[m] + (static_cast<int64_t>(kb) * kBK + g * 16) * 2;
+          bt.x[u][m][0] = *reinterpret_cast<const uint4 *>(src);
+          bt.x[u][m][1] = *reinterpret_cast<const uint4 *>(src + 16);
+        }
+      }
+    };
+    auto consume = [&](int kb0, const Batch &bt) {
+  #pragma unroll
+      for (int u = 0; u < kU; ++u) {
+        if (kb0 + u >= kb_end) break;  // uniform per wave
+        bf16x8 a0[TN], a1[TN];
+  #pragma unroll
+        for (int t = 0; t < TN; ++t) {
+          Pack16 lo, hi;
+          if (W8) {
+            const uint4 q = bt.w[u][t][0];
+            const uint2 c0 = cvt4_i8_bf16(q.x), c1 = cvt4_i8_bf16(q.y);
+            const uint2 c2 = cvt4_i8_bf16(q.z), c3 = cvt4_i8_bf16(q.w);
+            lo.u = make_uint4(c0.x, c0.y, c1.x, c1.y);
+            hi.u = make_uint4(c2.x, c2.y, c3.x, c3.y);
+          } else {
+            lo.u = bt.w[u][t][0];
+            hi.u = bt.w[u][t][kWL - 1];
+          }
+          a0[t] = lo.v;
+          a1[t] = hi.v;
+        }
+  #pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          Pack16 b0, b1;
+          b0.u = bt.x[u][m][0];
+          b1.u = bt.x[u][m][1];
+  #pragma unroll
+          for (int t = 0; t < TN; ++t) {
+            acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[t], b0.v, acc[t][m], 0, 0, 0);
+            acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[t], b1.v, acc[t][m], 0, 0, 0);
           }
         }
       }
-    }
-#pragma unroll
-    for (int u = 0; u < kU; ++u) {
-      const int kb = kb0 + u;
-      if (kb >= kb_end) break;  // uniform per wave
-      bf16x8 a0[TN], a1[TN];
-#pragma unroll
-      for (int t = 0; t < TN; ++t) {
-        Pack16 lo, hi;
-        if (W8) {
-          const uint4 q = wraw[u][t][0];
-          const uint2 c0 = cvt4_i8_bf16(q.x), c1 = cvt4_i8_bf16(q.y);
-          const uint2 c2 = cvt4_i8_bf16(q.z), c3 = cvt4_i8_bf16(q.w);
-          lo.u = make_uint4(c0.x, c0.y, c1.x, c1.y);
-          hi.u = make_uint4(c2.x, c2.y, c3.x, c3.y);
-        } else {
-          lo.u = wraw[u][t][0];
-          hi.u = wraw[u][t][W8 ? 0 : 1];
-        }
-        a0[t] = lo.v;
-        a1[t] = hi.v;
+    };
+    if (kb_begin < kb_end) {
+      Batch ba, bb;
+      issue(kb_begin, ba);
+      for (int kb0 = kb_begin; kb0 < kb_end; kb0 += 2 * kU) {
+        issue(kb0 + kU, bb);
+        consume(kb0, ba);
+        issue(kb0 + 2 * kU, ba);
+        consume(kb0 + kU, bb);
       }
-#pragma unroll
-      for (int m = 0; m < MT; ++m) {
-        Pack16 b0, b1;
-        b0.u = make_uint4(0, 0, 0, 0);
-        b1.u = make_uint4(0, 0, 0, 0);
-        if (xok[m]) {
-          const unsigned char *src = xrow[m] + (static_cast<int64_t>(kb) * kBK + g * 16) * 2;
-          b0.u = *reinterpret_cast<const uint4 *>(src);
-          b1.u = *reinterpret_cast<const uint4 *>(src + 16);
-        }
-#pragma unroll
+    }
+  } else {
+    // weights four K-blocks ahead, activations read from L2 where they are used (predicated: rows past M load nothing)
+    constexpr int kUOld = 4;
+    for (int kb0 = kb_begin; kb0 < kb_end; kb0 += kUOld) {
+      // issue the weight loads of up to kUOld K-blocks
+      uint4 wraw[kUOld][TN][W8 ? 1 : 2];
+  #pragma unroll
+      for (int u = 0; u < kUOld; ++u) {
+        const int kb = kb0 + u;
+  #pragma unroll
         for (int t = 0; t < TN; ++t) {
-          acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[t], b0.v, acc[t][m], 0, 0, 0);
-          acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[t], b1.v, acc[t][m], 0, 0, 0);
+          if (W8) {
+            wraw[u][t][0] = make_uint4(0, 0, 0, 0);
+            if (kb < kb_end && wok[t]) wraw[u][t][0] = load_nt_u4(wrow[t] + static_cast<int64_t>(kb) * 2048);
+          } else {
+            wraw[u][t][0] = make_uint4(0, 0, 0, 0);
+            wraw[u][t][W8 ? 0 : 1] = make_uint4(0, 0, 0, 0);
+            if (kb < kb_end && wok[t]) {
+              const unsigned char *src = wrow[t] + (static_cast<int64_t>(kb) * kBK + g * 16) * 2;
+              wraw[u][t][0] = load_nt_u4(src);
+              wraw[u][t][W8 ? 0 : 1] = load_nt_u4(src + 16);
+            }
+          }
+        }
+      }
+  #pragma unroll
+      for (int u = 0; u < kUOld; ++u) {
+        const int kb = kb0 + u;
+        if (kb >= kb_end) break;  // uniform per wave
+        bf16x8 a0[TN], a1[TN];
+  #pragma unroll
+        for (int t = 0; t < TN; ++t) {
+          Pack16 lo, hi;
+          if (W8) {
+            const uint4 q = wraw[u][t][0];
+            const uint2 c0 = cvt4_i8_bf16(q.x), c1 = cvt4_i8_bf16(q.y);
+            const uint2 c2 = cvt4_i8_bf16(q.z), c3 = cvt4_i8_bf16(q.w);
+            lo.u = make_uint4(c0.x, c0.y, c1.x, c1.y);
+            hi.u = make_uint4(c2.x, c2.y, c3.x, c3.y);
+          } else {
+            lo.u = wraw[u][t][0];
+            hi.u = wraw[u][t][W8 ? 0 : 1];
+          }
+          a0[t] = lo.v;
+          a1[t] = hi.v;
+        }
+  #pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          Pack16 b0, b1;
+          b0.u = make_uint4(0, 0, 0, 0);
+          b1.u = make_uint4(0, 0, 0, 0);
+          if (xok[m]) {
+            const unsigned char *src = xrow[m] + (static_cast<int64_t>(kb) * kBK + g * 16) * 2;
+            b0.u = *reinterpret_cast<const uint4 *>(src);
+            b1.u = *reinterpret_cast<const uint4 *>(src + 16);
+          }
+  #pragma unroll
+          for (int t = 0; t < TN; ++t) {
+            acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[t], b0.v, acc[t][m], 0, 0, 0);
+            acc[t][m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[t], b1.v, acc[t][m], 0, 0, 0);
+          }
         }
       }
     }
@@ -1046,12 +1134,19 @@ int launch_skinny(const GemmParams &p, hipStream_t stream) {
   else if (tiles16 >= 2 * 512) tn = 2;
   if (gemm_tuning().skinny_tn) tn = gemm_tuning().skinny_tn;
   const dim3 grid((tiles16 + tn - 1) / tn);
-#define TLF_SK(MT_, TN_) \
-  hipLaunchKernelGGL((skinny_gemm_kernel<MT_, TN_, W8>), grid, dim3(512), 0, stream, p)
-#define TLF_SK_TN(MT_)          \
-  if (tn == 4) TLF_SK(MT_, 4);  \
-  else if (tn == 2) TLF_SK(MT_, 2); \
-  else TLF_SK(MT_, 1)
+#define TLF_SK(MT_, TN_)                                                                                 \
+  if (MT_ == 1 && p.M <= 8)                                                                              \
+    hipLaunchKernelGGL((skinny_gemm_kernel<MT_, TN_, W8, MT_ == 1>), grid, dim3(512), 0, stream, p);     \
+  else                                                                                                   \
+    hipLaunchKernelGGL((skinny_gemm_kernel<MT_, TN_, W8, false>), grid, dim3(512), 0, stream, p)
+#define TLF_SK_TN(MT_)      \
+  if (tn == 4) {            \
+    TLF_SK(MT_, 4);         \
+  } else if (tn == 2) {     \
+    TLF_SK(MT_, 2);         \
+  } else {                  \
+    TLF_SK(MT_, 1);         \
+  }
   switch (mt) {
     case 1: TLF_SK_TN(1); break;
     case 2: TLF_SK_TN(2); break;
