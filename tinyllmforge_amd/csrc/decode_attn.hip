@@ -137,6 +137,9 @@ void paged_decode_kernel(const DecodeParams p) {
   const int head = w * group + n;
   const bool head_ok = n < group;
   const int max_ctx = p.max_blocks * p.block_size;  // a longer length would overrun the table
+  // fetched first: behind the scan their latency would sit in front of the first tile's loads
+  const float kscale = KV8 ? p.k_scale[w] : 1.0f;
+  const float vscale = KV8 ? p.v_scale[w] : 1.0f;
 
   // ---- 1. tiles per sequence -> exclusive prefix in LDS (block scan, chunks of kThreads)
   if (tid == 0) s_prefix[0] = 0;
@@ -167,15 +170,14 @@ void paged_decode_kernel(const DecodeParams p) {
   }
   const int total_tiles = carry;
 
-  // ---- 2. empty sequences get zeros (workgroup 0 owns that)
-  if (blockIdx.x == 0) {
-    for (int b = 0; b < p.batch; ++b) {
-      if (s_prefix[b + 1] == s_prefix[b]) {
-        if (tid == 0) *reinterpret_cast<int2 *>(p.meta + 2 * b) = make_int2(0, 0);
-        unsigned short *o = p.out + static_cast<int64_t>(b) * p.num_q_heads * kDh;
-        for (int i = tid * 8; i < p.num_q_heads * kDh; i += kThreads * 8)
-          *reinterpret_cast<uint4 *>(o + i) = make_uint4(0, 0, 0, 0);
-      }
+  // ---- 2. empty sequences get zeros: workgroup i looks after sequences i, i + G, ... (one workgroup walking
+  // the whole batch would finish its own share that much later, and the launch with it)
+  for (int b = blockIdx.x; b < p.batch; b += gridDim.x) {
+    if (s_prefix[b + 1] == s_prefix[b]) {
+      if (tid == 0) *reinterpret_cast<int2 *>(p.meta + 2 * b) = make_int2(0, 0);
+      unsigned short *o = p.out + static_cast<int64_t>(b) * p.num_q_heads * kDh;
+      for (int i = tid * 8; i < p.num_q_heads * kDh; i += kThreads * 8)
+        *reinterpret_cast<uint4 *>(o + i) = make_uint4(0, 0, 0, 0);
     }
   }
 
@@ -193,8 +195,6 @@ void paged_decode_kernel(const DecodeParams p) {
   const int64_t row_elems = static_cast<int64_t>(p.num_kv_heads) * kDh;
   unsigned short(*Ks)[kLdsRowK] = lds_k[w];
   unsigned short(*Vs)[kLdsRowV] = lds_v[w];
-  const float kscale = KV8 ? p.k_scale[w] : 1.0f;
-  const float vscale = KV8 ? p.v_scale[w] : 1.0f;
   const float scale_log2 = p.scale_log2 * kscale;
 
   // A segment = the part of one sequence that lies in this workgroup's share: sequence b, whose tiles are
