@@ -24,6 +24,8 @@
 // converted to fp16 once, when its tile is staged: exact for e4m3 rows, exact for bf16 rows between 6.1e-5
 // and 65504 in magnitude (smaller values keep 2^-24 absolute resolution, larger ones saturate at 65504:
 // the conversion rounds toward zero, which never produces an infinity).
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace tlf {
@@ -138,8 +140,8 @@ __device__ __forceinline__ void rescale16(floatx4 (&acc)[8], int d0, float alpha
   for (int e = 0; e < 16; ++e) acc[d0 + e / 4][e % 4] = t[e];
 }
 
-template <int CT, bool KV8>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))  // 256 registers: two workgroups per CU
+template <int CT, bool KV8, int NWV>
+__global__ __launch_bounds__(64 * NWV) __attribute__((amdgpu_waves_per_eu(2, 2)))  // 256 registers: two waves per SIMD
 void prefill_attn_kernel(const PrefillParams p) {
   __shared__ __attribute__((aligned(16))) unsigned short Ks[kBKV][kPRowK];  // bf16, rows in k_tile_row order
   __shared__ __attribute__((aligned(16))) unsigned short Vs[kBKV][kPRowV];  // fp16
@@ -158,7 +160,7 @@ void prefill_attn_kernel(const PrefillParams p) {
     seq = pair / static_cast<int>(gridDim.y);
   }
   const int group = p.num_q_heads / p.num_kv_heads;
-  const int bq = (64 * CT) / group;  // query rows per workgroup
+  const int bq = (16 * NWV * CT) / group;  // query rows per workgroup
   const int row0 = (gridDim.x - 1 - xt) * bq;
   const int q_begin = p.cu_q[seq];
   const int lq = p.cu_q[seq + 1] - q_begin;
@@ -200,11 +202,12 @@ void prefill_attn_kernel(const PrefillParams p) {
 
   // K/V tile loader: bf16 rows are 16 chunks of 16 B, e4m3 rows 8 chunks of 16 B.
   constexpr int kChunks = KV8 ? 8 : 16;
-  constexpr int kPasses = kBKV * kChunks / 256;
+  constexpr int kThreads = 64 * NWV;
+  constexpr int kPasses = kBKV * kChunks / kThreads;
   uint4 kreg[kPasses], vreg[kPasses];
   // Address arithmetic is kept off the vector ALU as far as possible (this kernel is VALU bound):
   // everything that depends on the thread only is computed once, the tile's share is scalar.
-  constexpr int kRowsPerPass = 256 / kChunks;
+  constexpr int kRowsPerPass = kThreads / kChunks;
   const int trow = tid / kChunks, ch = tid % kChunks;
   const int64_t k_thread = (static_cast<int64_t>(k_begin + trow) * p.k_stride + h * kPDh + ch * 8) * 2;
   const int64_t v_thread = (static_cast<int64_t>(k_begin + trow) * p.v_stride + h * kPDh + ch * 8) * 2;
@@ -448,14 +451,24 @@ extern "C" int tlf_varlen_prefill_attn(const void *q, int64_t q_stride, const vo
   p.num_cache_blocks = num_cache_blocks;
   p.scale_log2 = scale * kPLog2e;
   constexpr int CT = 2;
-  const int bq = (64 * CT) / group;
+  // 4 waves (128 (row, head) units, two workgroups per CU) or 8 waves (256 units, one workgroup per CU: half
+  // the K/V staging per unit; measured 4-5 % faster on sequences of 4096 and 8192 tokens, no faster on 1024 and
+  // below, where the longer row tiles waste more of the diagonal); TLF_PREFILL_WAVES overrides for tuning
+  static const int forced = [] {
+    const char *e = getenv("TLF_PREFILL_WAVES");
+    return e && atoi(e) == 4 ? 4 : e && atoi(e) == 8 ? 8 : 0;
+  }();
+  const int nwv = forced ? forced : max_seqlen_q >= 2048 ? 8 : 4;
+  const int bq = (16 * nwv * CT) / group;
   const dim3 grid((max_seqlen_q + bq - 1) / bq, num_kv_heads, num_seqs);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (paged && kv_dtype == TLF_KV_FP8_E4M3) {
     // the K scale is a per-head constant of the scores: fold it in on the device side per head
-    hipLaunchKernelGGL((prefill_attn_kernel<CT, true>), grid, dim3(256), 0, s, p);
+    if (nwv == 8) hipLaunchKernelGGL((prefill_attn_kernel<CT, true, 8>), grid, dim3(512), 0, s, p);
+    else hipLaunchKernelGGL((prefill_attn_kernel<CT, true, 4>), grid, dim3(256), 0, s, p);
   } else {
-    hipLaunchKernelGGL((prefill_attn_kernel<CT, false>), grid, dim3(256), 0, s, p);
+    if (nwv == 8) hipLaunchKernelGGL((prefill_attn_kernel<CT, false, 8>), grid, dim3(512), 0, s, p);
+    else hipLaunchKernelGGL((prefill_attn_kernel<CT, false, 4>), grid, dim3(256), 0, s, p);
   }
   return launch_status();
 }
