@@ -42,7 +42,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes per decode-attention launch on the default configs[1] workload, from two rocprofv3 --pmc runs
 # (FETCH_SIZE x 2.0 and WRITE_SIZE x 1.0 KiB per dispatch, factors taken from the 1 GiB copy probe), main + merge kernel
-DECODE_ATTN_TRAFFIC_BYTES = int((313290.6 + 2605.8) * 2.0 * 1024 + (5088.1 + 512.0) * 1024)
+DECODE_ATTN_TRAFFIC_BYTES = int((313290.1 + 2605.8) * 2.0 * 1024 + (5088.1 + 512.0) * 1024)
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 
 
