@@ -346,6 +346,10 @@ int tlf_paged_decode_attn(const void *q, int64_t q_stride,
  *     tlf_paged_decode_attn) and EVERY sequence reads its keys from them
  *     (layers/attention.py:99-100).
  * out: bf16 [total_q, Hq*Dh] contiguous.  max_seqlen_q bounds the grid.
+ * fp32 softmax and accumulation.  The P.V product runs in fp16: P (in [0, 1], 11 significant bits;
+ * flash-attn rounds it to one bf16, 8 bits) and V, which is converted to fp16 when its tile is staged
+ * - exact for e4m3 rows, exact for bf16 rows between 6.1e-5 and 65504 in magnitude; smaller values keep
+ * 2^-24 absolute resolution, larger ones saturate at 65504.
  * Dh == 128, Hq % Hkv == 0.
  */
 int tlf_varlen_prefill_attn(const void *q, int64_t q_stride,
