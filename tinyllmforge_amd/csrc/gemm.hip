@@ -1188,9 +1188,10 @@ inline bool plan_wstream(int M, int N, int K, int act, GemmPlan &g) {
   // Measured against the tiled plans on the Qwen3-8B projections with cold weights: a wide N (gate_up)
   // wins at every size up to 128 tokens (24 / 28 / 37 us at 32 / 64 / 128 tokens against 36 / 38 / 43);
   // a narrow N needs a split of K, whose activation traffic and partial sums grow with the token count:
-  // it wins up to 32 tokens (qkv 12 us against 15, o_proj 12 against 13.5) and, with a long K
-  // (down projection), up to 96 (17 / 22 / 25 us at 32 / 64 / 96 tokens against 26 / 27 / 28).
-  if (!t.ws_force && n_wg < 96 && !(M <= 32 || (ktiles >= 128 && M <= 96))) return false;
+  // it wins up to 32 tokens (qkv 12 us against 15, o_proj 12 against 13.5, down 18.7 against 19.8); above
+  // that the tiled plans with a split of K are faster (down projection, 48 / 64 / 96 tokens: 20.8 / 20.3 /
+  // 24.3 us against 23.8 / 23.1 / 28.9).
+  if (!t.ws_force && n_wg < 96 && M > 32) return false;
   if (act) {
     if (n_wg < 96) return false;
   } else {
@@ -1227,7 +1228,28 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
   const int ktiles = K / kBK;
   const int max_split = ktiles / 16 > 1 ? pow2_floor(ktiles / 16) : 1;
   int splits = 1;
-  if (M > 64 && M <= 224 && (N + 127) / 128 >= 128) {
+  const int n128 = (N + 127) / 128;
+  // Decode-size batches of int8 weights, from a sweep of every tile instance and split over the four Qwen3-8B
+  // projections on cold weights (us, this plan / the plan it replaced):
+  //  - moderate N, long K (down projection, 4096 x 12288): one M-tile as tall as the batch, 128 channels wide, K
+  //    split 8 ways (256 workgroups): 48 / 64 / 96 / 160 / 192 tokens 20.8 / 20.3 / 24.3 / 29.3 / 32.7 against
+  //    23.8 / 23.1 / 28.9 / 31.0 / 36.5;
+  //  - moderate N, K of 64 tiles, 48 tile columns and more (qkv, 6144 x 4096) above 160 tokens: the same tall
+  //    tile with K split 4 ways up to 224 tokens (176 / 192 / 208: 23.9 / 24.5 / 26.1 against 32.8 / 32.3 / 33.4),
+  //    two 128 x 128 tiles with K split in two above (256 tokens: 27.0 against 33.4);
+  //  - wide N (gate_up) from 193 to 256 tokens: 256 x 128 tile with eight waves (256 tokens: 60.8 against 71.2).
+  const bool tall_long_k = w8 && n128 < 128 && ktiles > 64 && M > 32 && M <= 208;
+  const bool mid_k64 = w8 && n128 < 128 && n128 >= 48 && ktiles <= 64 && ktiles % 4 == 0 && M > 160 && M <= 256;
+  if (tall_long_k || (mid_k64 && M <= 224)) {
+    g.bn = 128; g.bm = M <= 64 ? 64 : (M + 31) / 32 * 32; g.wn = 4;
+    g.stages = g.bm == 64 ? 4 : 3; g.occ = g.bm == 64 ? 3 : 2;
+    splits = tall_long_k ? 8 : 4;
+  } else if (mid_k64) {
+    g.bn = 128; g.bm = 128; g.stages = 3; g.occ = 2; g.wn = 4;
+    splits = 2;
+  } else if (w8 && n128 >= 128 && M > 192 && M <= 256 && tiles(256, 128) >= 160) {
+    g.bn = 256; g.bm = 128; g.stages = 3; g.occ = 2; g.wn = 8;
+  } else if (M > 64 && M <= 224 && (N + 127) / 128 >= 128) {
     // a decode-size batch against a very wide N (gate_up, LM head): one M-tile as tall as the
     // batch (rounded to 32 tokens), so nothing is padded to a power of two and W passes through
     // each CU once; four waves side by side along N.  Measured on 24576 x 4096 at M = 130:
