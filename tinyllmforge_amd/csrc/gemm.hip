@@ -1179,23 +1179,27 @@ inline bool plan_wstream(int M, int N, int K, int act, GemmPlan &g) {
   if (t.has_plan || M < t.ws_min_m || M > t.ws_max_m || M < 1 || act == 2) return false;
   // 128 or 96 channels per workgroup: whichever count of workgroups fills whole rounds of 256 CUs better
   auto fill = [](int wgs) { return static_cast<double>(wgs) / ((wgs + 255) / 256 * 256); };
+  const int ktiles = K / kBK;
+  const bool narrow = (N + 127) / 128 < 96;  // fewer than 96 workgroups of 128 channels: K has to be split
   int cols = 4;
   if (N >= 256 * 96 && fill((N + 95) / 96) > fill((N + 127) / 128) + 0.1) cols = 3;
+  if (narrow) cols = 3;
   if (t.ws_cols == 3 || t.ws_cols == 4) cols = t.ws_cols;
   const int n_wg = (N + cols * 32 - 1) / (cols * 32);
-  const int ktiles = K / kBK;
   int splits = 1;
   // Measured against the tiled plans on the Qwen3-8B projections with cold weights: a wide N (gate_up)
   // wins at every size up to 128 tokens (24 / 28 / 37 us at 32 / 64 / 128 tokens against 36 / 38 / 43);
   // a narrow N needs a split of K, whose activation traffic and partial sums grow with the token count:
-  // it wins up to 32 tokens (qkv 12 us against 15, o_proj 12 against 13.5, down 18.7 against 19.8); above
-  // that the tiled plans with a split of K are faster (down projection, 48 / 64 / 96 tokens: 20.8 / 20.3 /
-  // 24.3 us against 23.8 / 23.1 / 28.9).
-  if (!t.ws_force && n_wg < 96 && M > 32) return false;
+  // with 96-channel workgroups, K split 4 ways and one K part per workgroup (two for a long K) it wins up to
+  // 48 tokens (qkv 10.5 / 11.2 / 13.2 us at 17 / 32 / 48 tokens against 14.3 / 14.7 / 15.4 for the tiled plans,
+  // o_proj 9.5 / 9.7 / 11.6 against 13.1 / 13.5 / 14.2, down 16.0 / 16.9 at 17 / 32 against 25.8 / 25.9); above
+  // that the tiled plans with a split of K are faster.
+  if (!t.ws_force && narrow && M > (ktiles >= 128 ? 32 : 48)) return false;
   if (act) {
-    if (n_wg < 96) return false;
+    if (narrow) return false;
   } else {
     splits = (256 + n_wg / 2) / n_wg;
+    if (narrow && splits > 4) splits = 4;
     if (splits > ktiles / 8) splits = ktiles / 8;
     if (splits > 16) splits = 16;
     if (t.ws_splits) splits = t.ws_splits < ktiles ? t.ws_splits : ktiles;
@@ -1206,7 +1210,9 @@ inline bool plan_wstream(int M, int N, int K, int act, GemmPlan &g) {
   g.wstream = true;
   g.bn = cols * 32;
   g.bm = tm * 32;
-  int kg = ktiles % 2 == 0 && kt_per >= 4 ? 2 : 1;
+  // two K parts (two compute waves per SIMD) for a wide N from 33 tokens on and for a narrow N with a long K;
+  // elsewhere one part is 5-15 % faster (gate_up at 32 tokens 19.5 against 20.8 us, qkv 11.2 against 12.0)
+  int kg = ktiles % 2 == 0 && kt_per >= 4 && (narrow ? ktiles >= 128 : M > 32) ? 2 : 1;
   if (t.ws_kg && (t.ws_kg == 1 || ktiles % 2 == 0)) kg = t.ws_kg;
   g.stages = kg == 2 && tm >= 3 ? 3 : 4;
   g.occ = kg;
