@@ -1191,10 +1191,10 @@ inline bool plan_wstream(int M, int N, int K, int act, GemmPlan &g) {
   // wins at every size up to 128 tokens (24 / 28 / 37 us at 32 / 64 / 128 tokens against 36 / 38 / 43);
   // a narrow N needs a split of K, whose activation traffic and partial sums grow with the token count:
   // with 96-channel workgroups, K split 4 ways and one K part per workgroup (two for a long K) it wins up to
-  // 48 tokens (qkv 10.5 / 11.2 / 13.2 us at 17 / 32 / 48 tokens against 14.3 / 14.7 / 15.4 for the tiled plans,
-  // o_proj 9.5 / 9.7 / 11.6 against 13.1 / 13.5 / 14.2, down 16.0 / 16.9 at 17 / 32 against 25.8 / 25.9); above
-  // that the tiled plans with a split of K are faster.
-  if (!t.ws_force && narrow && M > (ktiles >= 128 ? 32 : 48)) return false;
+  // 80 tokens (qkv 10.5 / 11.2 / 14.4 / 16.2 us at 17 / 32 / 64 / 80 tokens against 14.3 / 14.7 / 16.3 / 17.3 for
+  // the tiled plans, o_proj 9.5 / 9.7 / 12.1 / 14.2 against 13.1 / 13.5 / 14.9 / 14.7) and, with a long K (down
+  // projection), up to 32 (16.0 / 16.9 at 17 / 32 against 25.8 / 25.9); above that the tiled plans are faster.
+  if (!t.ws_force && narrow && M > (ktiles >= 128 ? 32 : 80)) return false;
   if (act) {
     if (narrow) return false;
   } else {
