@@ -51,6 +51,11 @@ SHAPES = [  # (M, N, K)
     (150, 1024, 12288), (140, 6144, 4096), (90, 1040, 8320),
     # 256 x 256 tile with eight waves (ragged M and N) and the 256 x 128 tile with four waves side by side
     (2000, 24592, 192), (2050, 8208, 320), (1000, 6160, 192),
+    # W-streaming kernel with 5, 6 and 7 token tiles (wide N, 129 ... 224 tokens; ragged N), and a narrow N
+    # with K split across 96-channel workgroups
+    (150, 24592, 512), (190, 24576, 256), (220, 24592, 384), (70, 6144, 4096), (40, 4112, 1024),
+    # tall 128-channel tile with K split 8 ways (long K) and 4 ways (qkv shape above 160 tokens)
+    (100, 4096, 12288), (200, 4112, 8192), (180, 6144, 4096), (250, 6144, 4096),
 ]
 
 
@@ -66,7 +71,8 @@ def test_w8a16_gemm(M, N, K):
     check(got, exact, exact.to(BF), absdot)
 
 
-@pytest.mark.parametrize("M,N,K", [(5, 1024, 1024), (256, 4096, 4096), (130, 6144, 1024)])
+@pytest.mark.parametrize("M,N,K", [(5, 1024, 1024), (256, 4096, 4096), (130, 6144, 1024), (200, 24576, 512),
+                                   (60, 6144, 4096), (120, 4096, 12288), (8, 4096, 12288)])
 def test_w8a16_bit_exact_on_integer_activations(M, N, K):
     from tinyllmforge_amd import ops as P
     x = torch.randint(-4, 5, (M, K), generator=g(1)).to(BF)

@@ -1081,7 +1081,7 @@ struct GemmTuning {
   int skinny_max_m = kSkinnyMaxM;
   int skinny_tn = 0;
   int group_n = 0;
-  int ws_min_m = kSkinnyMaxM + 1, ws_max_m = 128;  // token range of the W-streaming kernel (int8 weights)
+  int ws_min_m = kSkinnyMaxM + 1, ws_max_m = 224;  // token range of the W-streaming kernel (int8 weights)
   int ws_splits = 0;                               // forced split of K for it
   int ws_kg = 0;                                   // forced K parts per workgroup (1 or 2)
   bool ws_force = false;                           // take it for every shape in its token range
@@ -1177,6 +1177,7 @@ struct GemmPlan {
 inline bool plan_wstream(int M, int N, int K, int act, GemmPlan &g) {
   const GemmTuning &t = gemm_tuning();
   if (t.has_plan || M < t.ws_min_m || M > t.ws_max_m || M < 1 || act == 2) return false;
+  if (M > 128 && !(N >= 256 * 96)) return false;  // 129 ... 224 tokens: 96-channel workgroups on a wide N only (below)
   // 128 or 96 channels per workgroup: whichever count of workgroups fills whole rounds of 256 CUs better
   auto fill = [](int wgs) { return static_cast<double>(wgs) / ((wgs + 255) / 256 * 256); };
   const int ktiles = K / kBK;
@@ -1184,6 +1185,10 @@ inline bool plan_wstream(int M, int N, int K, int act, GemmPlan &g) {
   int cols = 4;
   if (N >= 256 * 96 && fill((N + 95) / 96) > fill((N + 127) / 128) + 0.1) cols = 3;
   if (narrow) cols = 3;
+  // 160 ... 224 tokens: seven waves of up to 256 registers (96-channel workgroups, two K parts); measured on
+  // gate_up with cold weights 46.7 / 49.8 / 58.9 us at 160 / 192 / 224 tokens against 53.3 / 56.2 / 65.5 for the
+  // tiled plans, and no faster than the 256 x 128 tile at 256
+  if (M > 128) cols = 3;
   if (t.ws_cols == 3 || t.ws_cols == 4) cols = t.ws_cols;
   const int n_wg = (N + cols * 32 - 1) / (cols * 32);
   int splits = 1;
@@ -1214,7 +1219,8 @@ inline bool plan_wstream(int M, int N, int K, int act, GemmPlan &g) {
   // elsewhere one part is 5-15 % faster (gate_up at 32 tokens 19.5 against 20.8 us, qkv 11.2 against 12.0)
   int kg = ktiles % 2 == 0 && kt_per >= 4 && (narrow ? ktiles >= 128 : M > 32) ? 2 : 1;
   if (t.ws_kg && (t.ws_kg == 1 || ktiles % 2 == 0)) kg = t.ws_kg;
-  g.stages = kg == 2 && tm >= 3 ? 3 : 4;
+  if (tm > 4 && !(kg == 2 && cols == 3)) return false;  // the tall instances exist in that form only
+  g.stages = tm >= 7 ? 2 : kg == 2 && tm >= 3 ? 3 : 4;
   g.occ = kg;
   g.kgroups = kg;
   g.group_n = 1;
@@ -1442,6 +1448,8 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
       TLF_WS(1, 4, 8, 2, 4) TLF_WS(2, 4, 8, 2, 4) TLF_WS(3, 3, 4, 2, 4) TLF_WS(4, 3, 4, 2, 4)
       TLF_WS(1, 4, 8, 1, 3) TLF_WS(2, 4, 8, 1, 3) TLF_WS(3, 4, 8, 1, 3) TLF_WS(4, 4, 8, 1, 3)
       TLF_WS(1, 4, 8, 2, 3) TLF_WS(2, 4, 8, 2, 3) TLF_WS(3, 3, 8, 2, 3) TLF_WS(4, 3, 8, 2, 3)
+      TLF_WS(5, 3, 4, 2, 3) TLF_WS(6, 3, 4, 2, 3)  // seven waves: 256 registers each
+      TLF_WS(7, 2, 4, 2, 3)
 #undef TLF_WS
     }
   }
