@@ -56,6 +56,9 @@ SHAPES = [  # (M, N, K)
     (150, 24592, 512), (190, 24576, 256), (220, 24592, 384), (70, 6144, 4096), (40, 4112, 1024),
     # tall 128-channel tile with K split 8 ways (long K) and 4 ways (qkv shape above 160 tokens)
     (100, 4096, 12288), (200, 4112, 8192), (180, 6144, 4096), (250, 6144, 4096),
+    # 13 ... 16 tokens: W-streaming kernel on a wide N, a narrow N with K split and a long K; the skinny kernel
+    # stays for N <= 4096 with K <= 4096 (first rows of this list) and below 13 tokens
+    (16, 24592, 512), (13, 6144, 4096), (15, 4096, 12288), (12, 6144, 4096), (8, 24576, 512), (6, 4096, 4096),
 ]
 
 
@@ -72,7 +75,8 @@ def test_w8a16_gemm(M, N, K):
 
 
 @pytest.mark.parametrize("M,N,K", [(5, 1024, 1024), (256, 4096, 4096), (130, 6144, 1024), (200, 24576, 512),
-                                   (60, 6144, 4096), (120, 4096, 12288), (8, 4096, 12288)])
+                                   (60, 6144, 4096), (120, 4096, 12288), (8, 4096, 12288), (16, 6144, 4096),
+                                   (14, 24576, 512)])
 def test_w8a16_bit_exact_on_integer_activations(M, N, K):
     from tinyllmforge_amd import ops as P
     x = torch.randint(-4, 5, (M, K), generator=g(1)).to(BF)

@@ -1080,8 +1080,9 @@ struct GemmTuning {
   int plan[7] = {0, 0, 0, 0, 0, 1, 0};
   int skinny_max_m = kSkinnyMaxM;
   int skinny_tn = 0;
+  int skinny_pipe_m = -1;  // forced token limit of the skinny kernel's two-batch pipeline
   int group_n = 0;
-  int ws_min_m = kSkinnyMaxM + 1, ws_max_m = 224;  // token range of the W-streaming kernel (int8 weights)
+  int ws_min_m = 13, ws_max_m = 224;  // token range of the W-streaming kernel (int8 weights)
   int ws_splits = 0;                               // forced split of K for it
   int ws_kg = 0;                                   // forced K parts per workgroup (1 or 2)
   bool ws_force = false;                           // take it for every shape in its token range
@@ -1106,6 +1107,7 @@ inline const GemmTuning &gemm_tuning() {
       const int v = atoi(e);
       if (v == 1 || v == 2 || v == 4) g.skinny_tn = v;
     }
+    if (const char *e = getenv("TLF_GEMM_SKINNY_PIPE_M")) g.skinny_pipe_m = atoi(e);
     if (const char *e = getenv("TLF_GEMM_GROUP_N")) g.group_n = atoi(e) > 0 ? atoi(e) : 1;
     if (const char *e = getenv("TLF_GEMM_WSTREAM_M")) {
       int lo = 0, hi = 0;
@@ -1134,8 +1136,12 @@ int launch_skinny(const GemmParams &p, hipStream_t stream) {
   else if (tiles16 >= 2 * 512) tn = 2;
   if (gemm_tuning().skinny_tn) tn = gemm_tuning().skinny_tn;
   const dim3 grid((tiles16 + tn - 1) / tn);
+  // two batches in flight pay where a CU holds one workgroup or less (N <= 4096: o_proj 5.8 / 6.0 us at 6 / 8 tokens
+  // against 6.4 / 6.7, down 12.3 / 12.7 against 14.5 / 15.5) and up to 4 tokens everywhere; a wide N at 5 ... 8 tokens
+  // is 3-5 % faster on the plain loop
+  const int pipe_m = gemm_tuning().skinny_pipe_m >= 0 ? gemm_tuning().skinny_pipe_m : tiles16 <= 256 ? 8 : 4;
 #define TLF_SK(MT_, TN_)                                                                                 \
-  if (MT_ == 1 && p.M <= 8)                                                                              \
+  if (MT_ == 1 && p.M <= pipe_m)                                                                         \
     hipLaunchKernelGGL((skinny_gemm_kernel<MT_, TN_, W8, MT_ == 1>), grid, dim3(512), 0, stream, p);     \
   else                                                                                                   \
     hipLaunchKernelGGL((skinny_gemm_kernel<MT_, TN_, W8, false>), grid, dim3(512), 0, stream, p)
@@ -1178,6 +1184,9 @@ inline bool plan_wstream(int M, int N, int K, int act, GemmPlan &g) {
   const GemmTuning &t = gemm_tuning();
   if (t.has_plan || M < t.ws_min_m || M > t.ws_max_m || M < 1 || act == 2) return false;
   if (M > 128 && !(N >= 256 * 96)) return false;  // 129 ... 224 tokens: 96-channel workgroups on a wide N only (below)
+  // 13 ... 16 tokens, cold weights, W-streaming / skinny kernel at 16 tokens: qkv 10.5 / 11.8 us, gate_up 20.1 / 22.2,
+  // down 16.5 / 18.1, but o_proj (N = 4096, K = 4096: 43 workgroups x 4 splits) 9.3 / 7.8
+  if (M <= kSkinnyMaxM && !t.ws_force && N <= 4096 && K <= 4096) return false;
   // 128 or 96 channels per workgroup: whichever count of workgroups fills whole rounds of 256 CUs better
   auto fill = [](int wgs) { return static_cast<double>(wgs) / ((wgs + 255) / 256 * 256); };
   const int ktiles = K / kBK;
@@ -1378,7 +1387,9 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   p.act = act;
   p.amax = nullptr;
   p.amax_parts = 0;
-  if (M <= skinny_max_m()) {
+  GemmPlan g;
+  const bool wstream = W8 && plan_wstream(M, N, K, act, g);
+  if (M <= skinny_max_m() && !wstream) {
     p.k_per_split = K; p.splits = 1; p.m_tiles = 1; p.n_tiles = 1; p.group_n = 1;
     if (dry) {
       const int32_t skinny[8] = {0, 0, 0, 0, 1, 1, K, 1};  // tile 0 x 0 = the skinny kernel
@@ -1388,8 +1399,7 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
     if (act == 2) return TLF_E_UNSUPPORTED;  // the caller stages the logits and runs tlf_argmax
     return launch_skinny<W8>(p, stream);
   }
-  GemmPlan g;
-  if (!(W8 && plan_wstream(M, N, K, act, g))) {
+  if (!wstream) {
     g = plan_gemm(M, N, K, W8);
     plan_override(g, K);
   }
@@ -1592,7 +1602,6 @@ extern "C" int tlf_w8a16_pack_weight(const void *wq_rowmajor, void *packed, int3
 
 extern "C" size_t tlf_w8a16_gemm_workspace_bytes(int32_t M, int32_t N, int32_t K) {
   if (M <= 0 || N <= 0 || K <= 0 || K % kBK) return 0;
-  if (M <= skinny_max_m()) return 0;
   // fp32 partial sums of the plan's split of K (the larger of the int8 and the bf16 plan: both
   // entry points share this query); a tuning override may pick any split up to 16
   int splits = 16;
