@@ -274,6 +274,41 @@ int tlf_bf16_gemm_add_rmsnorm(const void *x, int64_t x_stride, const void *w, co
                               int32_t N, int32_t K, float eps, void *workspace,
                               size_t workspace_bytes, void *stream);
 
+/* qkv projection fused with what follows it in the attention block: replaces
+ * QKVParallelLinear.forward (layers/linear.py:82-83 through models/qwen3.py:78) followed by the
+ * q/k RMSNorm, RoPE and KV-cache store that tlf_qknorm_rope_store performs (models/qwen3.py:79-94,
+ * layers/attention.py:94-95).
+ *
+ *   qkv = bf16(scale[c] * sum_k x[t,k] wq[c,k])   [n, (Hq + 2 Hkv) * head_dim]   (bf16 entry: no scale, w bf16)
+ *   then exactly tlf_qknorm_rope_store(qkv, ...): same arguments, same outputs, same bits.
+ *
+ * When the plan for (n, (Hq + 2 Hkv) * head_dim, K) splits K across workgroups, the sum of the partial
+ * products, the norms, the rotation and the store are one kernel (qkv never goes to memory); otherwise qkv
+ * is staged in the workspace and the two kernels run back to back.
+ * workspace: tlf_gemm_qknorm_rope_store_workspace_bytes(n, (Hq + 2 Hkv) * head_dim, K) bytes, 256-byte
+ * aligned.  Other constraints as tlf_w8a16_gemm / tlf_bf16_gemm and tlf_qknorm_rope_store. */
+size_t tlf_gemm_qknorm_rope_store_workspace_bytes(int32_t M, int32_t N, int32_t K);
+int tlf_w8a16_gemm_qknorm_rope_store(const void *x, int64_t x_stride, const void *wq, const float *scale,
+                                     const void *q_norm_weight, const void *k_norm_weight, float eps,
+                                     const int64_t *positions, const float *cos_sin, int32_t max_pos,
+                                     void *q_out, void *k_out, void *v_out,
+                                     void *k_cache, void *v_cache, const int32_t *slot_mapping,
+                                     int64_t num_slots, int32_t kv_dtype,
+                                     const float *k_scale, const float *v_scale,
+                                     int32_t n, int32_t num_q_heads, int32_t num_kv_heads,
+                                     int32_t head_dim, int32_t K,
+                                     void *workspace, size_t workspace_bytes, void *stream);
+int tlf_bf16_gemm_qknorm_rope_store(const void *x, int64_t x_stride, const void *w,
+                                    const void *q_norm_weight, const void *k_norm_weight, float eps,
+                                    const int64_t *positions, const float *cos_sin, int32_t max_pos,
+                                    void *q_out, void *k_out, void *v_out,
+                                    void *k_cache, void *v_cache, const int32_t *slot_mapping,
+                                    int64_t num_slots, int32_t kv_dtype,
+                                    const float *k_scale, const float *v_scale,
+                                    int32_t n, int32_t num_q_heads, int32_t num_kv_heads,
+                                    int32_t head_dim, int32_t K,
+                                    void *workspace, size_t workspace_bytes, void *stream);
+
 /* LM head fused with the greedy sample: replaces ParallelLMHead.forward's product
  * (layers/embed_head.py:63) followed by Sampler.forward's greedy branch (layers/sampler.py:13-14,21)
  * when every temperature of the batch is 0.

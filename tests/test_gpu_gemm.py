@@ -187,6 +187,67 @@ def test_row_projection_with_add_rmsnorm_equals_the_two_kernels(M, N, K, w8, pat
         assert rel <= 2e-3, rel
 
 
+@pytest.mark.parametrize("n,Hq,Hkv,K,w8,fp8,want_kv,path", [
+    (48, 32, 8, 4096, True, False, False, "fused"),      # 8B qkv shape, W-streaming kernel with K split 4 ways
+    (200, 32, 8, 4096, True, False, False, "fused"),     # tall tile with K split 4 ways
+    (30, 64, 8, 5120, True, True, False, "fused"),       # 32B shape, e4m3 cache
+    (20, 16, 8, 1024, True, False, True, "fused"),       # config-1 shape, K rows also returned
+    (70, 16, 8, 2048, False, False, False, "fused"),     # bf16 weights, split plan
+    (120, 32, 8, 4096, True, False, False, "staged"),    # no split: projection staged, two kernels
+    (3, 32, 8, 4096, True, True, False, "staged"),       # skinny kernel
+    (700, 16, 8, 1024, False, False, True, "staged")])   # prefill-size batch
+def test_qkv_projection_with_qknorm_rope_store_equals_the_two_calls(n, Hq, Hkv, K, w8, fp8, want_kv, path):
+    """qkv projection together with the q/k norm, RoPE and KV-cache store that follow it: bit-identical to the
+    GEMM entry point followed by tlf_qknorm_rope_store on both routes -- the fused split-K reduce kernel
+    ("fused") and plans without a split ("staged") -- for q, the returned K/V rows and the caches."""
+    import ctypes
+    from tinyllmforge_amd import _lib, ops as P
+    Dh, maxpos, nblk, bs = 128, 4096, 4, 256
+    N = (Hq + 2 * Hkv) * Dh
+    plan = (ctypes.c_int32 * 8)()
+    assert _lib.load().tlf_gemm_plan(n, N, K, int(w8), plan) == 0
+    assert (plan[5] > 1) == (path == "fused"), list(plan)
+    x = torch.randn(n, K, generator=g(n + 21)).to(BF).to(DEV)
+    if w8:
+        w, scale = make_w8(N, K, N + 5)
+        scale = (scale / 8).to(DEV)
+        w = P.pack_w8(w.to(DEV))
+        qkv = P.w8a16_linear(x, w, scale)
+    else:
+        w, scale = (torch.randn(N, K, generator=g(N + 5)) / K ** 0.5).to(BF).to(DEV), None
+        qkv = P.bf16_linear(x, w)
+    tab = O.rope_table(Dh, maxpos, 1e6).to(DEV)
+    pos = torch.randint(0, maxpos, (n,), generator=g(n)).to(DEV)
+    if n > 2:
+        pos[2] = maxpos          # outside the table: passed through unrotated on both routes
+    qw = (1 + 0.2 * torch.randn(Dh, generator=g(7))).to(BF).to(DEV)
+    kw = (1 + 0.2 * torch.randn(Dh, generator=g(8))).to(BF).to(DEV)
+    slots = torch.randperm(nblk * bs, generator=g(9))[:n].to(torch.int32)
+    if n > 2:
+        slots[1] = -1
+    slots = slots.to(DEV)
+    cache_dtype = torch.float8_e4m3fn if fp8 else BF
+    def caches():
+        kc = torch.randn(nblk, bs, Hkv, Dh, generator=g(10)).to(DEV).to(cache_dtype)
+        vc = torch.randn(nblk, bs, Hkv, Dh, generator=g(11)).to(DEV).to(cache_dtype)
+        return kc, vc
+    ks = (torch.rand(Hkv, generator=g(12)) * 0.05 + 0.03).to(DEV) if fp8 else None
+    vs = (torch.rand(Hkv, generator=g(13)) * 0.05 + 0.03).to(DEV) if fp8 else None
+    kc2, vc2 = caches()
+    q2, k2, v2 = P.qknorm_rope_store(qkv, qw, kw, 1e-6, pos, tab, Hq, Hkv, Dh, kc2, vc2, slots, ks, vs, want_kv=want_kv)
+    kc1, vc1 = caches()
+    q1, k1, v1 = P.linear_qknorm_rope_store(x, w, scale, qw, kw, 1e-6, pos, tab, Hq, Hkv, Dh, kc1, vc1, slots, ks, vs,
+                                            want_kv=want_kv)
+    assert torch.equal(q1.view(torch.int16), q2.view(torch.int16))
+    assert torch.equal(kc1.view(torch.uint8), kc2.view(torch.uint8))
+    assert torch.equal(vc1.view(torch.uint8), vc2.view(torch.uint8))
+    if want_kv:
+        assert torch.equal(k1.view(torch.int16), k2.view(torch.int16))
+        assert torch.equal(v1.view(torch.int16), v2.view(torch.int16))
+    else:
+        assert k1 is None and v1 is None
+
+
 @pytest.mark.parametrize("M,N,K", [(4, 4112, 256), (40, 4112, 512), (130, 9008, 256), (300, 20000, 128), (256, 151936, 64)])
 def test_lm_head_with_greedy_sample_equals_gemm_then_argmax(M, N, K):
     """LM head + argmax in one call (no logits stored) against the two entry points it replaces, on logits

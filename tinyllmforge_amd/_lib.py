@@ -46,6 +46,11 @@ SIGNATURES = {
     "tlf_gemm_plan": (c_int32, [_I32, _I32, _I32, _I32, _P]),
     "tlf_gemm_add_rmsnorm_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
     "tlf_gemm_argmax_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
+    "tlf_gemm_qknorm_rope_store_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
+    "tlf_w8a16_gemm_qknorm_rope_store": (c_int32, [_P, _I64, _P, _P, _P, _P, _F, _P, _P, _I32, _P, _P, _P, _P, _P, _P,
+                                                   _I64, _I32, _P, _P, _I32, _I32, _I32, _I32, _I32, _P, _SZ, _P]),
+    "tlf_bf16_gemm_qknorm_rope_store": (c_int32, [_P, _I64, _P, _P, _P, _F, _P, _P, _I32, _P, _P, _P, _P, _P, _P,
+                                                  _I64, _I32, _P, _P, _I32, _I32, _I32, _I32, _I32, _P, _SZ, _P]),
     "tlf_bf16_gemm_argmax": (c_int32, [_P, _I64, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),
     "tlf_w8a16_gemm_add_rmsnorm": (c_int32, [_P, _I64, _P, _P, _P, _P, _P, _P, _I32, _I32, _I32, _F, _P, _SZ, _P]),
     "tlf_bf16_gemm_add_rmsnorm": (c_int32, [_P, _I64, _P, _P, _P, _P, _P, _I32, _I32, _I32, _F, _P, _SZ, _P]),

@@ -4,6 +4,7 @@
 #include <mutex>
 
 #include "common.h"
+#include "qknorm_rope.h"
 
 namespace tlf {
 
@@ -115,97 +116,17 @@ __global__ __launch_bounds__(256) void rope_kernel(
 }
 
 // --------------------------------------------------------------------------
-// Fused q/k RMSNorm + RoPE + KV-cache store over the qkv projection
-// (reference op sequence: tinyvllm/models/qwen3.py:79-94, layers/attention.py:94-95).
-// 16 lanes own one head (8 dims each); lanes j < 8 hold the first half of the
-// head, lanes j >= 8 the second, so the RoPE partner of lane j is lane j ^ 8.
-__global__ __launch_bounds__(256) void qknorm_rope_store_kernel(
-    const unsigned short *__restrict__ qkv, int64_t qkv_stride,
-    const unsigned short *__restrict__ qw, const unsigned short *__restrict__ kw, float eps,
-    const int64_t *__restrict__ positions, const float *__restrict__ cos_sin, int32_t max_pos,
-    unsigned short *__restrict__ q_out, unsigned short *__restrict__ k_out,
-    unsigned short *__restrict__ v_out, unsigned char *__restrict__ k_cache,
-    unsigned char *__restrict__ v_cache, const int32_t *__restrict__ slot_mapping,
-    int64_t num_slots, int32_t kv_dtype, const float *__restrict__ k_scale,
-    const float *__restrict__ v_scale, int32_t num_q_heads, int32_t num_kv_heads) {
+// Fused q/k RMSNorm + RoPE + KV-cache store over the qkv projection (qknorm_rope.h): one workgroup handles
+// 16 heads of one token, 16 lanes per head.
+__global__ __launch_bounds__(256) void qknorm_rope_store_kernel(const unsigned short *__restrict__ qkv,
+                                                                int64_t qkv_stride, const QkRopeStoreArgs a) {
   constexpr int kDh = 128;
   const int64_t tok = blockIdx.x;
   const int head = blockIdx.y * 16 + threadIdx.x / 16;
   const int j = threadIdx.x % 16;
-  const int heads = num_q_heads + 2 * num_kv_heads;
-  if (head >= heads) return;  // whole 16-lane groups leave together
-  const unsigned short *src = qkv + tok * qkv_stride + head * kDh + j * 8;
-  const uint4 raw = *reinterpret_cast<const uint4 *>(src);
-  const bool is_q = head < num_q_heads;
-  const bool is_k = !is_q && head < num_q_heads + num_kv_heads;
-  const int kvh = is_q ? 0 : (is_k ? head - num_q_heads : head - num_q_heads - num_kv_heads);
-  int64_t slot = -1;
-  if (!is_q && slot_mapping != nullptr) {
-    slot = slot_mapping[tok];
-    if (slot >= num_slots) slot = -1;
-  }
-  uint4 outp = raw;
-  if (is_q || is_k) {
-    float v[8];
-    unpack8(raw, v);
-    float ss = 0.f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) ss = fmaf(v[i], v[i], ss);
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
-    const float inv = 1.0f / sqrtf(ss / static_cast<float>(kDh) + eps);
-    float w[8];
-    unpack8(*reinterpret_cast<const uint4 *>((is_q ? qw : kw) + j * 8), w);
-    float nrm[8], other[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float nn = bf16_bits_to_float(float_to_bf16_bits(__fmul_rn(v[i], inv)));
-      nrm[i] = bf16_bits_to_float(float_to_bf16_bits(__fmul_rn(nn, w[i])));
-    }
-#pragma unroll
-    for (int i = 0; i < 8; ++i) other[i] = __shfl_xor(nrm[i], 8, 64);
-    const int64_t pos = positions[tok];
-    const bool pos_ok = pos >= 0 && pos < max_pos;
-    const float *cs = cos_sin + (pos_ok ? pos : 0) * kDh;
-    const int cj = (j % 8) * 8;
-    float o[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float co = cs[cj + i];
-      const float si = cs[64 + cj + i];
-      // lanes j < 8: cos*x1 - sin*x2 ; lanes j >= 8: cos*x2 + sin*x1
-      const float a = __fmul_rn(co, nrm[i]);
-      const float b = __fmul_rn(si, other[i]);
-      o[i] = (j < 8) ? __fsub_rn(a, b) : __fadd_rn(a, b);
-      if (!pos_ok) o[i] = nrm[i];
-    }
-    outp = pack8(o);
-  }
-  if (is_q) {
-    *reinterpret_cast<uint4 *>(q_out + tok * static_cast<int64_t>(num_q_heads) * kDh + head * kDh +
-                               j * 8) = outp;
-    return;
-  }
-  const int64_t row_elems = static_cast<int64_t>(num_kv_heads) * kDh;
-  unsigned short *lin = is_k ? k_out : v_out;
-  if (lin != nullptr) *reinterpret_cast<uint4 *>(lin + tok * row_elems + kvh * kDh + j * 8) = outp;
-  if (slot < 0) return;
-  unsigned char *cache = is_k ? k_cache : v_cache;
-  if (kv_dtype == TLF_KV_BF16) {
-    *reinterpret_cast<uint4 *>(cache + (slot * row_elems + kvh * kDh + j * 8) * 2) = outp;
-  } else {
-    float f[8];
-    unpack8(outp, f);
-    const float s = (is_k ? k_scale : v_scale)[kvh];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) f[i] = fminf(fmaxf(f[i] / s, -448.0f), 448.0f);
-    int lo = 0, hi = 0;
-    lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[0], f[1], lo, false);
-    lo = __builtin_amdgcn_cvt_pk_fp8_f32(f[2], f[3], lo, true);
-    hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[4], f[5], hi, false);
-    hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
-    *reinterpret_cast<int2 *>(cache + slot * row_elems + kvh * kDh + j * 8) = make_int2(lo, hi);
-  }
+  if (head >= a.num_q_heads + 2 * a.num_kv_heads) return;  // whole 16-lane groups leave together
+  const uint4 raw = *reinterpret_cast<const uint4 *>(qkv + tok * qkv_stride + head * kDh + j * 8);
+  qknorm_rope_store_piece(raw, tok, head, j, a);
 }
 
 // --------------------------------------------------------------------------
@@ -477,21 +398,16 @@ extern "C" int tlf_rope(const int64_t *positions, const void *q, int64_t q_strid
   return launch_status();
 }
 
-extern "C" int tlf_qknorm_rope_store(const void *qkv, int64_t qkv_stride, const void *q_norm_weight,
-                                     const void *k_norm_weight, float eps, const int64_t *positions,
-                                     const float *cos_sin, int32_t max_pos, void *q_out,
-                                     void *k_out, void *v_out, void *k_cache, void *v_cache,
-                                     const int32_t *slot_mapping, int64_t num_slots,
-                                     int32_t kv_dtype, const float *k_scale, const float *v_scale,
-                                     int32_t n, int32_t num_q_heads, int32_t num_kv_heads,
-                                     int32_t head_dim, void *stream) {
-  if (n == 0) return TLF_OK;
-  if (!qkv || !q_norm_weight || !k_norm_weight || !positions || !cos_sin || !q_out)
-    return TLF_E_NULL;
+int tlf::check_qk_rope_store_args(const void *q_norm_weight, const void *k_norm_weight,
+                                  const int64_t *positions, const float *cos_sin, int32_t max_pos,
+                                  const void *q_out, const void *k_out, const void *v_out,
+                                  const void *k_cache, const void *v_cache, const int32_t *slot_mapping,
+                                  int64_t num_slots, int32_t kv_dtype, const float *k_scale,
+                                  const float *v_scale, int32_t n, int32_t num_q_heads,
+                                  int32_t num_kv_heads, int32_t head_dim) {
+  if (!q_norm_weight || !k_norm_weight || !positions || !cos_sin || !q_out) return TLF_E_NULL;
   if (head_dim != 128) return TLF_E_UNSUPPORTED;
   if (n < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || max_pos <= 0) return TLF_E_SHAPE;
-  const int heads = num_q_heads + 2 * num_kv_heads;
-  if (qkv_stride < static_cast<int64_t>(heads) * head_dim) return TLF_E_SHAPE;
   if (slot_mapping != nullptr) {
     if (!k_cache || !v_cache) return TLF_E_NULL;
     if (num_slots <= 0) return TLF_E_SHAPE;
@@ -502,18 +418,37 @@ extern "C" int tlf_qknorm_rope_store(const void *qkv, int64_t qkv_stride, const 
     }
     if (!aligned16(k_cache) || !aligned16(v_cache)) return TLF_E_ALIGN;
   }
-  if (!aligned16(qkv) || qkv_stride % 8 || !aligned16(q_out) || !aligned16(q_norm_weight) ||
-      !aligned16(k_norm_weight) || (k_out && !aligned16(k_out)) || (v_out && !aligned16(v_out)))
+  if (!aligned16(q_out) || !aligned16(q_norm_weight) || !aligned16(k_norm_weight) ||
+      (k_out && !aligned16(k_out)) || (v_out && !aligned16(v_out)))
     return TLF_E_ALIGN;
+  return TLF_OK;
+}
+
+extern "C" int tlf_qknorm_rope_store(const void *qkv, int64_t qkv_stride, const void *q_norm_weight,
+                                     const void *k_norm_weight, float eps, const int64_t *positions,
+                                     const float *cos_sin, int32_t max_pos, void *q_out,
+                                     void *k_out, void *v_out, void *k_cache, void *v_cache,
+                                     const int32_t *slot_mapping, int64_t num_slots,
+                                     int32_t kv_dtype, const float *k_scale, const float *v_scale,
+                                     int32_t n, int32_t num_q_heads, int32_t num_kv_heads,
+                                     int32_t head_dim, void *stream) {
+  if (n == 0) return TLF_OK;
+  if (!qkv) return TLF_E_NULL;
+  const int rc = check_qk_rope_store_args(q_norm_weight, k_norm_weight, positions, cos_sin, max_pos, q_out, k_out,
+                                          v_out, k_cache, v_cache, slot_mapping, num_slots, kv_dtype, k_scale,
+                                          v_scale, n, num_q_heads, num_kv_heads, head_dim);
+  if (rc != TLF_OK) return rc;
+  const int heads = num_q_heads + 2 * num_kv_heads;
+  if (qkv_stride < static_cast<int64_t>(heads) * head_dim) return TLF_E_SHAPE;
+  if (!aligned16(qkv) || qkv_stride % 8) return TLF_E_ALIGN;
+  const QkRopeStoreArgs a{static_cast<const unsigned short *>(q_norm_weight),
+                          static_cast<const unsigned short *>(k_norm_weight), eps, positions, cos_sin, max_pos,
+                          static_cast<unsigned short *>(q_out), static_cast<unsigned short *>(k_out),
+                          static_cast<unsigned short *>(v_out), static_cast<unsigned char *>(k_cache),
+                          static_cast<unsigned char *>(v_cache), slot_mapping, num_slots, kv_dtype, k_scale,
+                          v_scale, num_q_heads, num_kv_heads};
   hipLaunchKernelGGL(qknorm_rope_store_kernel, dim3(n, (heads + 15) / 16), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const unsigned short *>(qkv),
-                     qkv_stride, static_cast<const unsigned short *>(q_norm_weight),
-                     static_cast<const unsigned short *>(k_norm_weight), eps, positions, cos_sin,
-                     max_pos, static_cast<unsigned short *>(q_out),
-                     static_cast<unsigned short *>(k_out), static_cast<unsigned short *>(v_out),
-                     static_cast<unsigned char *>(k_cache), static_cast<unsigned char *>(v_cache),
-                     slot_mapping, num_slots, kv_dtype, k_scale, v_scale, num_q_heads,
-                     num_kv_heads);
+                     static_cast<hipStream_t>(stream), static_cast<const unsigned short *>(qkv), qkv_stride, a);
   return launch_status();
 }
 

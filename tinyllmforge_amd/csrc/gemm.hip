@@ -33,6 +33,7 @@
 #include <stdlib.h>
 
 #include "common.h"
+#include "qknorm_rope.h"
 
 namespace tlf {
 
@@ -740,6 +741,41 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmParams p) 
   *reinterpret_cast<uint2 *>(p.y + i4 * 4) = st;
 }
 
+// What follows the qkv projection in the decoder is the q/k RMSNorm, RoPE and the KV-cache store
+// (reference: tinyvllm/models/qwen3.py:79-94, layers/attention.py:94-95).  When K was split across
+// workgroups this kernel is the sum of the partials and that step in one pass: the 16 lanes of a head first
+// form h = bf16(sum_k partial_k * scale), exactly what splitk_reduce_kernel would store, and go on from
+// there as the kernel that reads the projection from memory does (same bits).
+template <bool W8>
+__global__ __launch_bounds__(256) void splitk_reduce_qknorm_rope_store_kernel(const GemmParams p,
+                                                                              const QkRopeStoreArgs a) {
+  const int64_t tok = blockIdx.x;
+  const int head = blockIdx.y * 16 + threadIdx.x / 16;
+  const int j = threadIdx.x % 16;
+  if (head >= a.num_q_heads + 2 * a.num_kv_heads) return;  // whole 16-lane groups leave together
+  const int n = head * 128 + j * 8;
+  const int64_t mn = static_cast<int64_t>(p.M) * p.N;
+  const float *src = p.partial + tok * p.N + n;
+  float4 s0 = *reinterpret_cast<const float4 *>(src);
+  float4 s1 = *reinterpret_cast<const float4 *>(src + 4);
+#pragma unroll 4
+  for (int k = 1; k < p.splits; ++k) {
+    const float4 t0 = *reinterpret_cast<const float4 *>(src + k * mn);
+    const float4 t1 = *reinterpret_cast<const float4 *>(src + k * mn + 4);
+    s0.x += t0.x; s0.y += t0.y; s0.z += t0.z; s0.w += t0.w;
+    s1.x += t1.x; s1.y += t1.y; s1.z += t1.z; s1.w += t1.w;
+  }
+  if (W8) {
+    const float4 c0 = *reinterpret_cast<const float4 *>(p.scale + n);
+    const float4 c1 = *reinterpret_cast<const float4 *>(p.scale + n + 4);
+    s0.x *= c0.x; s0.y *= c0.y; s0.z *= c0.z; s0.w *= c0.w;
+    s1.x *= c1.x; s1.y *= c1.y; s1.z *= c1.z; s1.w *= c1.w;
+  }
+  const uint4 raw = make_uint4(pack_bf16x2(s0.x, s0.y), pack_bf16x2(s0.z, s0.w), pack_bf16x2(s1.x, s1.y),
+                               pack_bf16x2(s1.z, s1.w));
+  qknorm_rope_store_piece(raw, tok, head, j, a);
+}
+
 // What follows a row-parallel projection in the decoder (o_proj, down_proj) is the residual add and
 // an RMSNorm (reference: tinyvllm/models/qwen3.py:163-166 after linear.py:181-183).  When K was
 // split across workgroups the projection's value only exists after the partial sums are added, so
@@ -1374,7 +1410,7 @@ template <bool W8>
 int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *scale, void *y,
                 int32_t M, int32_t N, int32_t K, void *workspace, size_t workspace_bytes,
                 hipStream_t stream, int32_t *plan_out = nullptr, int32_t act = 0,
-                const NormTail *tail = nullptr) {
+                const NormTail *tail = nullptr, const QkRopeStoreArgs *qk = nullptr) {
   const bool dry = plan_out != nullptr;
   GemmParams p;
   p.x = static_cast<const unsigned char *>(x);
@@ -1517,6 +1553,12 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
 #undef TLF_TAIL
       return launch_status();
     }
+    if (qk) {  // likewise: N = (Hq + 2 Hkv) * 128
+      hipLaunchKernelGGL((splitk_reduce_qknorm_rope_store_kernel<W8>),
+                         dim3(static_cast<unsigned>(M), static_cast<unsigned>((N / 128 + 15) / 16)), dim3(256), 0,
+                         stream, p, *qk);
+      return launch_status();
+    }
     const int64_t total4 = static_cast<int64_t>(M) * N / 4;
     hipLaunchKernelGGL((splitk_reduce_kernel<W8>), dim3(static_cast<unsigned>((total4 + 255) / 256)),
                        dim3(256), 0, stream, p);
@@ -1568,6 +1610,29 @@ int launch_gemm_add_rmsnorm(const void *x, int64_t x_stride, const void *w, cons
   if (rc != TLF_OK) return rc;
   return tlf_add_rmsnorm(ws, tail.residual, tail.weight, tail.y, tail.residual_out, M, N, tail.eps,
                          stream);
+}
+
+// qkv projection followed by q/k RMSNorm + RoPE + KV-cache store, the same way: a plan that splits K ends in
+// the fused reduce kernel, every other plan stages the projection at the head of the workspace.
+template <bool W8>
+int launch_gemm_qknorm_rope_store(const void *x, int64_t x_stride, const void *w, const float *scale,
+                                  const QkRopeStoreArgs &a, int32_t M, int32_t N, int32_t K, void *workspace,
+                                  size_t workspace_bytes, hipStream_t stream) {
+  int32_t plan[8];
+  int rc = launch_gemm<W8>(nullptr, K, nullptr, nullptr, nullptr, M, N, K, nullptr, 0, nullptr, plan);
+  if (rc != TLF_OK) return rc;
+  if (plan[5] > 1)
+    return launch_gemm<W8>(x, x_stride, w, scale, nullptr, M, N, K, workspace, workspace_bytes, stream, nullptr, 0,
+                           nullptr, &a);
+  const size_t tmp_bytes = align256(static_cast<size_t>(M) * N * 2);
+  if (!workspace || workspace_bytes < tmp_bytes || (reinterpret_cast<uintptr_t>(workspace) & 255u))
+    return TLF_E_WORKSPACE;
+  unsigned char *ws = static_cast<unsigned char *>(workspace);
+  rc = launch_gemm<W8>(x, x_stride, w, scale, ws, M, N, K, ws + tmp_bytes, workspace_bytes - tmp_bytes, stream);
+  if (rc != TLF_OK) return rc;
+  return tlf_qknorm_rope_store(ws, N, a.qw, a.kw, a.eps, a.positions, a.cos_sin, a.max_pos, a.q_out, a.k_out,
+                               a.v_out, a.k_cache, a.v_cache, a.slot_mapping, a.num_slots, a.kv_dtype, a.k_scale,
+                               a.v_scale, M, a.num_q_heads, a.num_kv_heads, 128, stream);
 }
 
 inline int check_gemm_args(const void *x, int64_t x_stride, const void *w, const void *y, int32_t M,
@@ -1733,4 +1798,70 @@ extern "C" int tlf_bf16_gemm_argmax(const void *x, int64_t x_stride, const void 
   }
   return launch_gemm<false>(x, x_stride, w, nullptr, token_ids, M, N, K, workspace, workspace_bytes, st,
                             nullptr, 2);
+}
+
+extern "C" size_t tlf_gemm_qknorm_rope_store_workspace_bytes(int32_t M, int32_t N, int32_t K) {
+  if (M <= 0 || N <= 0 || K <= 0 || K % kBK) return 0;
+  return align256(static_cast<size_t>(M) * N * 2) + align256(tlf_w8a16_gemm_workspace_bytes(M, N, K));
+}
+
+namespace {
+template <bool W8>
+int gemm_qknorm_rope_store_entry(const void *x, int64_t x_stride, const void *w, const float *scale,
+                                 const void *q_norm_weight, const void *k_norm_weight, float eps,
+                                 const int64_t *positions, const float *cos_sin, int32_t max_pos, void *q_out,
+                                 void *k_out, void *v_out, void *k_cache, void *v_cache,
+                                 const int32_t *slot_mapping, int64_t num_slots, int32_t kv_dtype,
+                                 const float *k_scale, const float *v_scale, int32_t n, int32_t num_q_heads,
+                                 int32_t num_kv_heads, int32_t head_dim, int32_t K, void *workspace,
+                                 size_t workspace_bytes, void *stream) {
+  if (n == 0) return TLF_OK;
+  int rc = check_qk_rope_store_args(q_norm_weight, k_norm_weight, positions, cos_sin, max_pos, q_out, k_out, v_out,
+                                    k_cache, v_cache, slot_mapping, num_slots, kv_dtype, k_scale, v_scale, n,
+                                    num_q_heads, num_kv_heads, head_dim);
+  if (rc != TLF_OK) return rc;
+  const int64_t N64 = (static_cast<int64_t>(num_q_heads) + 2 * num_kv_heads) * head_dim;
+  if (N64 > (1 << 30)) return TLF_E_SHAPE;
+  const int32_t N = static_cast<int32_t>(N64);
+  rc = check_gemm_args(x, x_stride, w, q_out, n, N, K);
+  if (rc != TLF_OK) return rc;
+  if (W8) {
+    if (!scale) return TLF_E_NULL;
+    if (reinterpret_cast<uintptr_t>(scale) & 15u) return TLF_E_ALIGN;
+  }
+  const QkRopeStoreArgs a{static_cast<const unsigned short *>(q_norm_weight),
+                          static_cast<const unsigned short *>(k_norm_weight), eps, positions, cos_sin, max_pos,
+                          static_cast<unsigned short *>(q_out), static_cast<unsigned short *>(k_out),
+                          static_cast<unsigned short *>(v_out), static_cast<unsigned char *>(k_cache),
+                          static_cast<unsigned char *>(v_cache), slot_mapping, num_slots, kv_dtype, k_scale,
+                          v_scale, num_q_heads, num_kv_heads};
+  return launch_gemm_qknorm_rope_store<W8>(x, x_stride, w, scale, a, n, N, K, workspace, workspace_bytes,
+                                           static_cast<hipStream_t>(stream));
+}
+}  // namespace
+
+extern "C" int tlf_w8a16_gemm_qknorm_rope_store(
+    const void *x, int64_t x_stride, const void *wq, const float *scale, const void *q_norm_weight,
+    const void *k_norm_weight, float eps, const int64_t *positions, const float *cos_sin, int32_t max_pos,
+    void *q_out, void *k_out, void *v_out, void *k_cache, void *v_cache, const int32_t *slot_mapping,
+    int64_t num_slots, int32_t kv_dtype, const float *k_scale, const float *v_scale, int32_t n,
+    int32_t num_q_heads, int32_t num_kv_heads, int32_t head_dim, int32_t K, void *workspace,
+    size_t workspace_bytes, void *stream) {
+  return gemm_qknorm_rope_store_entry<true>(x, x_stride, wq, scale, q_norm_weight, k_norm_weight, eps, positions,
+                                            cos_sin, max_pos, q_out, k_out, v_out, k_cache, v_cache, slot_mapping,
+                                            num_slots, kv_dtype, k_scale, v_scale, n, num_q_heads, num_kv_heads,
+                                            head_dim, K, workspace, workspace_bytes, stream);
+}
+
+extern "C" int tlf_bf16_gemm_qknorm_rope_store(
+    const void *x, int64_t x_stride, const void *w, const void *q_norm_weight, const void *k_norm_weight,
+    float eps, const int64_t *positions, const float *cos_sin, int32_t max_pos, void *q_out, void *k_out,
+    void *v_out, void *k_cache, void *v_cache, const int32_t *slot_mapping, int64_t num_slots,
+    int32_t kv_dtype, const float *k_scale, const float *v_scale, int32_t n, int32_t num_q_heads,
+    int32_t num_kv_heads, int32_t head_dim, int32_t K, void *workspace, size_t workspace_bytes,
+    void *stream) {
+  return gemm_qknorm_rope_store_entry<false>(x, x_stride, w, nullptr, q_norm_weight, k_norm_weight, eps, positions,
+                                             cos_sin, max_pos, q_out, k_out, v_out, k_cache, v_cache, slot_mapping,
+                                             num_slots, kv_dtype, k_scale, v_scale, n, num_q_heads, num_kv_heads,
+                                             head_dim, K, workspace, workspace_bytes, stream);
 }

@@ -183,6 +183,18 @@ class QKVParallelLinear(ColumnParallelLinear):
         self.num_kv_heads = self.total_num_kv_heads
         super().__init__(hidden_size, (self.num_heads + 2 * self.num_kv_heads) * head_size, bias)
 
+    def forward_qknorm_rope_store(self, x: torch.Tensor, q_norm, k_norm, positions, cos_sin, k_cache, v_cache,
+                                  slot_mapping, k_scale, v_scale, want_kv: bool):
+        """``ops.qknorm_rope_store(self(x), ...)`` (models/qwen3.py:78-94 + layers/attention.py:94-95) behind
+        one call; ``q_norm`` / ``k_norm`` are the RMSNorm modules.  Returns ``(q, k, v)``."""
+        tail = (q_norm.weight.data, k_norm.weight.data, q_norm.eps, positions, cos_sin, self.num_heads,
+                self.num_kv_heads, self.head_size, k_cache, v_cache, slot_mapping, k_scale, v_scale)
+        if self.bias is not None:
+            return ops.qknorm_rope_store(self.forward(x), *tail, want_kv=want_kv)
+        if self.is_quantized:
+            return ops.linear_qknorm_rope_store(x, self.pack_().qpacked, self.qscale, *tail, want_kv=want_kv)
+        return ops.linear_qknorm_rope_store(x, self.weight.data, None, *tail, want_kv=want_kv)
+
     def shard_rows(self, shard_id=None):
         assert shard_id in ("q", "k", "v")
         q_size, kv_size = self.num_heads * self.head_size, self.num_kv_heads * self.head_size

@@ -41,20 +41,21 @@ class QWen3Attention(nn.Module):
     def forward(self, positions: torch.Tensor, hidden_states: torch.Tensor, residual=None, norm=None):
         """``o_proj(attention(...))``; with ``norm`` (the RMSNorm that follows, and its ``residual``) the
         projection and the add-norm are one call and ``(normed, residual)`` is returned."""
-        qkv = self.qkv_proj(hidden_states)
         if self.fused:
             ctx = get_context()
             attn = self.attn
             has_cache = attn.has_cache()
             # prefill without a prefix hit attends over this step's own K/V rows
             want_kv = ctx.is_prefill and ctx.block_tables is None
-            q, k, v = ops.qknorm_rope_store(
-                qkv, self.q_norm.weight.data, self.k_norm.weight.data, self.q_norm.eps, positions,
-                self.rotary_emb.cos_sin_cache, self.num_heads, self.num_kv_heads, self.head_dim,
+            # projection, q/k norm, RoPE and cache store in one call (one kernel fewer when the projection's
+            # plan splits K across workgroups, which is the rule at decode sizes)
+            q, k, v = self.qkv_proj.forward_qknorm_rope_store(
+                hidden_states, self.q_norm, self.k_norm, positions, self.rotary_emb.cos_sin_cache,
                 attn.k_cache if has_cache else None, attn.v_cache if has_cache else None,
-                ctx.slot_mapping if has_cache else None, attn.k_scale, attn.v_scale, want_kv=want_kv)
+                ctx.slot_mapping if has_cache else None, attn.k_scale, attn.v_scale, want_kv)
             o = attn(q, k, v, kv_stored=True)
         else:
+            qkv = self.qkv_proj(hidden_states)
             q, k, v = qkv.split([self.q_size, self.kv_size, self.kv_size], dim=-1)
             q = self.q_norm(q.view(-1, self.num_heads, self.head_dim)).view(-1, self.q_size)
             k = self.k_norm(k.view(-1, self.num_kv_heads, self.head_dim)).view(-1, self.kv_size)

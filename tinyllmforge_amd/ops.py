@@ -357,6 +357,50 @@ def linear_add_rms_norm(x, w, scale, residual, norm_weight, eps):
     return y.view(shape), r.view(shape)
 
 
+def linear_qknorm_rope_store(x, w, scale, q_weight, k_weight, eps, positions, cos_sin, num_q_heads, num_kv_heads,
+                             head_dim, k_cache=None, v_cache=None, slot_mapping=None, k_scale=None, v_scale=None,
+                             want_kv=False):
+    """``qknorm_rope_store(linear(x), ...)`` behind one call: ``w`` int8 with ``scale`` (weight-only int8) or
+    bf16 with ``scale=None``.  Returns ``(q, k, v)`` with the bits of the two separate calls."""
+    lib = _lib.load()
+    w8 = scale is not None
+    if w8:
+        w = _packed(w)
+        _need(scale, torch.float32, "scale")
+    else:
+        _need(w, BF16, "w")
+        assert w.is_contiguous()
+    _need(x, BF16, "x"); _need(positions, torch.int64, "positions")
+    assert x.stride(-1) == 1
+    x2 = x.reshape(-1, x.shape[-1])
+    n, K = x2.shape
+    N = (num_q_heads + 2 * num_kv_heads) * head_dim
+    assert w.shape[0] == N
+    q = torch.empty(n, num_q_heads * head_dim, dtype=BF16, device=x.device)
+    k = v = None
+    if want_kv:
+        k = torch.empty(n, num_kv_heads * head_dim, dtype=BF16, device=x.device)
+        v = torch.empty(n, num_kv_heads * head_dim, dtype=BF16, device=x.device)
+    has_cache = k_cache is not None and k_cache.numel() > 0 and slot_mapping is not None
+    kvd = kv_dtype_code(k_cache) if has_cache else KV_BF16
+    num_slots = (k_cache.numel() // (num_kv_heads * head_dim)) if has_cache else 0
+    ws = _workspace(lib.tlf_gemm_qknorm_rope_store_workspace_bytes(n, N, K), x.device, "gemm")
+    tail = (q_weight.data_ptr(), k_weight.data_ptr(), float(eps), positions.data_ptr(), cos_sin.data_ptr(),
+            cos_sin.shape[0], q.data_ptr(), k.data_ptr() if k is not None else None,
+            v.data_ptr() if v is not None else None, k_cache.data_ptr() if has_cache else None,
+            v_cache.data_ptr() if has_cache else None, slot_mapping.data_ptr() if has_cache else None, num_slots,
+            kvd, k_scale.data_ptr() if k_scale is not None else None,
+            v_scale.data_ptr() if v_scale is not None else None, n, num_q_heads, num_kv_heads, head_dim, K,
+            ws.data_ptr(), ws.numel(), _stream())
+    if w8:
+        check(lib.tlf_w8a16_gemm_qknorm_rope_store(x2.data_ptr(), x2.stride(0), w.data_ptr(), scale.data_ptr(),
+                                                   *tail), "tlf_w8a16_gemm_qknorm_rope_store")
+    else:
+        check(lib.tlf_bf16_gemm_qknorm_rope_store(x2.data_ptr(), x2.stride(0), w.data_ptr(), *tail),
+              "tlf_bf16_gemm_qknorm_rope_store")
+    return q, k, v
+
+
 # ------------------------------------------------------------------ a3
 def paged_decode_attention(q, k_cache, v_cache, context_lens, block_tables, scale,
                            k_scale=None, v_scale=None):
