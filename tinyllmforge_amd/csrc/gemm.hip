@@ -75,6 +75,19 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
                                               int n0, int wn, int wm, int r, int kg, int split) {
   // Epilogue.  acc[i][j][v]: token m = m0 + wm*WM + j*32 + r,
   // channel n = n0 + wn*WN + i*32 + (v/4)*8 + kg*4 + (v%4).
+  // The channel scales of this lane's registers, fetched once: read where they are used, each load sits behind
+  // the previous store (the compiler cannot rule out that y and scale overlap) and the epilogue becomes a chain
+  // of load -> multiply -> store round trips, 32 of them for a 256-token tile.
+  float4 sc[TN][4];
+  if (W8 && p.splits == 1) {
+#pragma unroll
+    for (int i = 0; i < TN; ++i)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int n = n0 + wn * WN + i * 32 + q * 8 + kg * 4;
+        sc[i][q] = n < p.N ? *reinterpret_cast<const float4 *>(p.scale + n) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+  }
   if (p.act == 2) {
     // LM head + greedy sample (reference: tinyvllm/layers/embed_head.py:63, sampler.py:13-14,21): the
     // logits are never stored.  A token's channels of this wave sit in the registers of lanes r and
@@ -95,7 +108,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
 #pragma unroll
           for (int e = 0; e < 4; ++e) o[e] = acc[i][j][q * 4 + e];
           if (W8) {
-            const float4 s = *reinterpret_cast<const float4 *>(p.scale + n);
+            const float4 s = sc[i][q];
             o[0] *= s.x; o[1] *= s.y; o[2] *= s.z; o[3] *= s.w;
           }
 #pragma unroll
@@ -112,19 +125,29 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
     }
     return;
   }
+  // bf16 results leave as 16-byte stores: lanes r and r + 32 hold the same token and alternate groups of 4
+  // channels, so one half-wave exchange (v_permlane32_swap) hands lane r the 8 consecutive channels 16 h ..
+  // 16 h + 7 and lane r + 32 the next 8 -- half the store instructions, rows written 32 bytes at a time.
+  auto swap_pairs = [](uint2 &a, uint2 &b) {
+    // before: lane kg holds channel groups (2 h) and (2 h + 1) of its own; after: lane 0 holds group 2 h of
+    // both lanes (channels 0..7 of the 16), lane 1 group 2 h + 1 of both (channels 8..15)
+    auto rx = __builtin_amdgcn_permlane32_swap(a.x, b.x, false, false);
+    auto ry = __builtin_amdgcn_permlane32_swap(a.y, b.y, false, false);
+    a = make_uint2(rx[0], ry[0]);
+    b = make_uint2(rx[1], ry[1]);
+  };
 #pragma unroll
   for (int j = 0; j < TM; ++j) {
     const int m = m0 + wm * WM + j * 32 + r;
-    if (m >= p.M) continue;
+    const bool m_ok = m < p.M;
 #pragma unroll
     for (int i = 0; i < TN; ++i) {
       if (p.act == 1) {
         // channels come in groups of 16 = 8 gate rows then the 8 matching up rows, so this lane's
         // registers q = 0, 2 hold gate values and q = 1, 3 the up values of the same 4 channels
+        uint2 st[2];
 #pragma unroll
         for (int q = 0; q < 4; q += 2) {
-          const int n = n0 + wn * WN + i * 32 + q * 8 + kg * 4;  // first gate row of the four
-          if (n >= p.N) continue;
           float gt[4], up[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
@@ -132,8 +155,7 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
             up[e] = acc[i][j][(q + 1) * 4 + e];
           }
           if (W8) {
-            const float4 sg = *reinterpret_cast<const float4 *>(p.scale + n);
-            const float4 su = *reinterpret_cast<const float4 *>(p.scale + n + 8);
+            const float4 sg = sc[i][q], su = sc[i][q + 1];
             gt[0] *= sg.x; gt[1] *= sg.y; gt[2] *= sg.z; gt[3] *= sg.w;
             up[0] *= su.x; up[1] *= su.y; up[2] *= su.z; up[3] *= su.w;
           }
@@ -142,34 +164,48 @@ __device__ __forceinline__ void gemm_epilogue(const GemmParams &p, floatx16 (&ac
           for (int e = 0; e < 4; ++e)  // both factors rounded to bf16 first, as the unfused sequence does
             o[e] = silu_mul_bf16(bf16_bits_to_float(float_to_bf16_bits(gt[e])),
                                  bf16_bits_to_float(float_to_bf16_bits(up[e])));
-          uint2 st;
-          st.x = pack_bf16x2(o[0], o[1]);
-          st.y = pack_bf16x2(o[2], o[3]);
-          const int c = (n0 + wn * WN + i * 32) / 2 + (q / 2) * 8 + kg * 4;  // output channel
-          *reinterpret_cast<uint2 *>(p.y + static_cast<int64_t>(m) * (p.N / 2) + c) = st;
+          st[q / 2] = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
+        }
+        // this lane: output channels c0 + kg*4 .. (q = 0) and c0 + 8 + kg*4 .. (q = 2) of the 16 of this tile
+        swap_pairs(st[0], st[1]);
+        const int nfirst = n0 + wn * WN + i * 32;
+        if (m_ok && nfirst + kg * 16 < p.N) {  // lane r + 32 stores what came from the tile's second 16 rows
+          const int c = nfirst / 2 + kg * 8;
+          *reinterpret_cast<uint4 *>(p.y + static_cast<int64_t>(m) * (p.N / 2) + c) =
+              make_uint4(st[0].x, st[0].y, st[1].x, st[1].y);
         }
         continue;
       }
+      if (p.splits > 1) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = n0 + wn * WN + i * 32 + q * 8 + kg * 4;
+          if (!m_ok || n >= p.N) continue;  // N % 4 == 0, so a group of 4 is all in or all out
+          float *dst = p.partial + (static_cast<int64_t>(split) * p.M + m) * p.N + n;
+          *reinterpret_cast<float4 *>(dst) =
+              make_float4(acc[i][j][q * 4], acc[i][j][q * 4 + 1], acc[i][j][q * 4 + 2], acc[i][j][q * 4 + 3]);
+        }
+        continue;
+      }
+      uint2 st[4];
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int n = n0 + wn * WN + i * 32 + q * 8 + kg * 4;
-        if (n >= p.N) continue;  // N % 4 == 0, so a group of 4 is all in or all out
         float o[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) o[e] = acc[i][j][q * 4 + e];
-        if (p.splits > 1) {
-          float *dst = p.partial + (static_cast<int64_t>(split) * p.M + m) * p.N + n;
-          *reinterpret_cast<float4 *>(dst) = make_float4(o[0], o[1], o[2], o[3]);
-        } else {
-          if (W8) {
-            const float4 s = *reinterpret_cast<const float4 *>(p.scale + n);
-            o[0] *= s.x; o[1] *= s.y; o[2] *= s.z; o[3] *= s.w;
-          }
-          uint2 st;
-          st.x = pack_bf16x2(o[0], o[1]);
-          st.y = pack_bf16x2(o[2], o[3]);
-          *reinterpret_cast<uint2 *>(p.y + static_cast<int64_t>(m) * p.N + n) = st;
+        if (W8) {
+          const float4 s = sc[i][q];
+          o[0] *= s.x; o[1] *= s.y; o[2] *= s.z; o[3] *= s.w;
         }
+        st[q] = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
+      }
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        swap_pairs(st[2 * h], st[2 * h + 1]);
+        const int n = n0 + wn * WN + i * 32 + h * 16 + kg * 8;  // N % 16 == 0: 16 channels are all in or all out
+        if (m_ok && n < p.N)
+          *reinterpret_cast<uint4 *>(p.y + static_cast<int64_t>(m) * p.N + n) =
+              make_uint4(st[2 * h].x, st[2 * h].y, st[2 * h + 1].x, st[2 * h + 1].y);
       }
     }
   }
