@@ -205,6 +205,106 @@ def test_c1_eager_equals_graph_and_rerun_hits_prefix_cache(llm_c1, golden):
     assert [x[0] for x in a] == [x[0] for x in c]
 
 
+def forced_steps(llm, prompts, tokens):
+    """Run ``prompts`` through the engine's runner for ``len(tokens[0])`` steps, feeding ``tokens[s][step]``
+    after every step whatever the model chose.  Returns the last-token hidden states and whole logit rows of
+    every step and the number of prompt tokens served from cached blocks."""
+    from tinyllmforge_amd.engine.sequence import Sequence
+    from tinyllmforge_amd.sampling_params import SamplingParams
+    from tinyllmforge_amd.utils.context import get_context, reset_context
+    runner, sch = llm.model_runner, llm.scheduler
+    steps = len(tokens[0])
+    sp = SamplingParams(temperature=0.0, max_tokens=steps, ignore_eos=True)
+    seqs0 = [Sequence(p, sp) for p in prompts]
+    for s in seqs0:
+        sch.add(s)
+    out, cached, paged = [], 0, None
+    for step in range(steps):
+        seqs, is_prefill = sch.schedule()
+        assert seqs == seqs0 and is_prefill == (step == 0)
+        if is_prefill:
+            cached = sum(s.num_cached_tokens for s in seqs)
+            ids, pos = runner.prepare_prefill(seqs)
+            paged = get_context().block_tables is not None
+        else:
+            ids, pos = runner.prepare_decode(seqs)
+        hidden = runner.run_hidden(ids, pos, is_prefill)
+        logits = runner.model.compute_logits(hidden).float().cpu()
+        if is_prefill:
+            hidden = hidden[(get_context().cu_seqlens_q[1:] - 1).long()]
+        out.append((hidden.cpu(), logits))
+        reset_context()
+        sch.postprocess(seqs, [t[step] for t in tokens])
+    assert sch.is_finished()
+    return out, cached, paged
+
+
+def test_c1_prefix_hit_run_teacher_forced_against_the_dense_run(llm_c1):
+    """The engine-level prefix-hit path at config 1, all 8 steps: the same prompts run once with a dense prefill
+    (nothing cached) and once with their first block served from cached blocks (paged prefill over 256 cached +
+    40 fresh tokens per sequence, then decode over the same blocks), both fed the SAME tokens.  The two runs
+    differ only in the tiles the prefill kernel walks, so their hidden states and whole logit rows must agree
+    to rounding noise at every step - a wiring error in the paged-prefill path (wrong block, offset or mask
+    alignment) is O(1) and cannot hide behind a near-tie of the sampled token."""
+    from oracle import ops as O
+    from tinyllmforge_amd import SamplingParams
+    prompts = [p + p + p[:40] for p in c1_prompts()]          # 296 tokens: one full (hashable) block + a tail
+    forget_prefix_cache(llm_c1)
+    free = llm_c1.generate(prompts, SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))
+    tokens = [o["token_ids"] for o in free]
+    forget_prefix_cache(llm_c1)
+    dense, cached, paged = forced_steps(llm_c1, prompts, tokens)
+    assert cached == 0 and paged is False
+    hit, cached, paged = forced_steps(llm_c1, prompts, tokens)  # the blocks of the run before are still hashed
+    assert cached == 4 * 256 and paged is True
+    worst_h = worst_u = 0.0
+    for step, ((hd, ld), (hh, lh)) in enumerate(zip(dense, hit)):
+        h_l2 = ((hh.float() - hd.float()).norm(dim=-1) / hd.float().norm(dim=-1)).max().item()
+        ulps = ((lh - ld).abs().amax(dim=-1) / O.bf16_ulp(ld.abs().amax(dim=-1))).max().item()
+        worst_h, worst_u = max(worst_h, h_l2), max(worst_u, ulps)
+        assert h_l2 <= 3e-2 and ulps <= 3.0, (step, h_l2, ulps)
+        top = ld.topk(2, dim=-1)
+        clear = (top.values[:, 0] - top.values[:, 1]) > 2 * O.bf16_ulp(top.values[:, 0])
+        assert torch.equal(lh.argmax(-1)[clear], top.indices[clear, 0]), step
+    print(f"prefix-hit vs dense run, 8 steps: hidden rel L2 <= {worst_h:.2e}, logit rows within {worst_u:.2f} ulp of the row max")
+
+
+def test_reference_bench_recipe_under_the_tinyvllm_name():
+    """The reference's bench.py (lines 31, 39-56) as its author wrote it, against this package: imported as
+    ``tinyvllm``, ``LLM(model, enforce_eager=False, max_model_len=4096)``, prompts and output lengths from the
+    same ``random`` recipe (8 of its 256 sequences), ``generate(prompts, sampling_params, use_tqdm=False)`` with
+    the script's own temperature 0.6, then greedy.  Every request must run to its ``max_tokens`` and the greedy
+    run must reproduce itself token for token."""
+    from bench import e2e_workload
+    from tinyllmforge_amd import dropin
+    dropin.install()
+    try:
+        from tinyvllm import LLM, SamplingParams
+        prompts, max_tokens = e2e_workload(8)
+        max_tokens = [min(m, 160) for m in max_tokens]
+        llm = LLM("qwen3-0.6b", enforce_eager=False, max_model_len=4096)
+        try:
+            sps = [SamplingParams(temperature=0.6, ignore_eos=True, max_tokens=m) for m in max_tokens]
+            llm.generate(["Benchmark: "] if llm.tokenizer is not None else [[1, 2, 3]], SamplingParams(max_tokens=4), use_tqdm=False)
+            out = llm.generate(prompts, sps, use_tqdm=False)
+            assert [len(o["token_ids"]) for o in out] == max_tokens
+            vocab = llm.config.hf_config.vocab_size
+            assert all(0 <= t < vocab for o in out for t in o["token_ids"])
+            greedy = [SamplingParams(temperature=0.0, ignore_eos=True, max_tokens=m) for m in max_tokens]
+            forget_prefix_cache(llm)                        # both greedy runs prefill every token (dense kernel)
+            a = [o["token_ids"] for o in llm.generate(prompts, greedy, use_tqdm=False)]
+            forget_prefix_cache(llm)
+            b = [o["token_ids"] for o in llm.generate(prompts, greedy, use_tqdm=False)]
+            assert a == b and [len(x) for x in a] == max_tokens
+            assert llm.last_stats["decode_steps"] == max(max_tokens) - 1
+            import tinyvllm.layers.attention as A
+            assert isinstance(llm.model_runner.model.model.layers[0].self_attn.attn, A.Attention)
+        finally:
+            llm.exit()
+    finally:
+        dropin.uninstall()
+
+
 def test_fused_lm_head_argmax_gives_the_tokens_of_logits_then_sampler(llm_c1):
     """All-greedy batches sample through the fused LM head + argmax; with it switched off the same batch goes
     through logits and the sampler kernel.  Same tokens, prefill (4 last rows) and graph decode alike."""

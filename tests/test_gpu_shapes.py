@@ -6,6 +6,10 @@
   bf16 linears, on sequences of the benchmark's recipe: graph decode == eager decode, fused == unfused layer
   path, step statistics, block manager clean at the end; its KV pool is larger than 2 GiB per layer side and
   the blocks in use are taken from its far end.
+* The Qwen3-32B-shaped engine at its own depth (config 5: 64 layers, hidden 5120, 64 / 8 heads, intermediate
+  25600), W8A16 linears, e4m3 KV cache, prompts of 2048 ... 8192 tokens of which two share a 1024-token prefix held
+  in cached blocks: graph decode == eager decode, fused == unfused layer path, prefix hits counted, block
+  manager clean.
 * Two-layer decoders at the 8B and 32B WIDTHS against the CPU oracle, teacher-forced: final hidden state and
   whole logit rows at every step.  The 32B-width run uses W8A16 linears, an e4m3 KV cache with a different
   scale per KV head and layer, and a 1024-token prefix held in cached blocks (config 5).
@@ -132,6 +136,71 @@ def test_8b_engine_graph_equals_eager_and_fused_equals_unfused(quantization):
                 layer.self_attn.fused = True
         assert c == [x[:6] for x in a], "fused and unfused layer paths differ"
         assert not bm.used_block_ids and len(bm.free_block_ids) == nblk
+    finally:
+        close(llm)
+
+
+# ----------------------------------------------------------------------------- config 5: the 32B engine
+def test_32b_engine_64_layers_cached_prefix_graph_equals_eager_and_fused_equals_unfused():
+    """configs[4] at its own depth and width: 64 layers, hidden 5120, 64 query / 8 KV heads, intermediate 25600,
+    W8A16 linears, e4m3 KV cache with a different scale per KV head.  Four prompts of 2048 ... 8192 tokens, two of
+    them behind a 1024-token prefix that a first request left in cached blocks, 8 greedy tokens each: the prefill
+    steps run the paged kernel over e4m3 rows (a prefix hit sends every sequence of the step there), the decode
+    steps replay the hipGraph.  The same requests decoded eagerly, and again through the unfused layer path
+    (projection, then norm / RoPE / store as separate kernels), must give the same tokens."""
+    from tinyllmforge_amd import LLM, SamplingParams
+    nblk = 160
+    hkv = 8
+    k_scale = [(1.0 + 0.1 * h) / 16 for h in range(hkv)]
+    v_scale = [(1.4 - 0.05 * h) / 16 for h in range(hkv)]
+    llm = LLM("qwen3-32b", enforce_eager=False, max_model_len=8704, max_num_batched_tokens=16384, max_num_seqs=8,
+              quantization="w8a16", kv_cache_dtype="fp8_e4m3", kv_k_scale=k_scale, kv_v_scale=v_scale,
+              num_kvcache_blocks=nblk, seed=0)
+    try:
+        runner, bm = llm.model_runner, llm.scheduler.block_manager
+        hf = llm.config.hf_config
+        assert (hf.num_hidden_layers, hf.hidden_size, hf.num_attention_heads, hf.num_key_value_heads,
+                hf.intermediate_size) == (64, 5120, 64, 8, 25600)
+        assert runner.kv_cache.shape == (2, 64, nblk, 256, 8, 128) and runner.kv_cache.dtype == torch.float8_e4m3fn
+        assert len(runner.model.model.layers) == 64
+        shared = random_prompts((1024,), seed=31, vocab=10000)[0]
+        bodies = random_prompts((3000 - 1024, 2048, 8192 - 1024, 5000), seed=32, vocab=10000)
+        prompts = [shared + bodies[0], bodies[1], shared + bodies[2], bodies[3]]
+        assert [len(p) for p in prompts] == [3000, 2048, 8192, 5000]
+        sp = SamplingParams(temperature=0.0, ignore_eos=True, max_tokens=8)
+        one = SamplingParams(temperature=0.0, ignore_eos=True, max_tokens=1)
+
+        def run(n_tokens=8):
+            forget_prefix_cache(llm)
+            llm.generate([shared + [1, 2, 3]], one)            # leaves the prefix in four hashed blocks
+            out = llm.generate(prompts, SamplingParams(temperature=0.0, ignore_eos=True, max_tokens=n_tokens))
+            st = dict(llm.last_stats)
+            assert st["cached_prompt_tokens"] == 2048, st      # 1024 tokens for each of the two sequences behind the prefix
+            assert not bm.used_block_ids and len(bm.free_block_ids) == nblk
+            return [o["token_ids"] for o in out], st
+
+        a, st = run()
+        assert st["decode_steps"] == 7 and st["prefill_steps"] >= 2       # 18,240 prompt tokens: two prefill steps
+        assert all(len(x) == 8 for x in a) and all(0 <= t < hf.vocab_size for x in a for t in x)
+        assert len({tuple(x) for x in a}) == 4
+        runner.enforce_eager = True
+        try:
+            b, _ = run()
+        finally:
+            runner.enforce_eager = False
+        assert a == b, "graph decode and eager decode differ"
+        runner.enforce_eager = True
+        runner.model.model.fused = False
+        for layer in runner.model.model.layers:
+            layer.self_attn.fused = False
+        try:
+            c, _ = run(4)
+        finally:
+            runner.enforce_eager = False
+            runner.model.model.fused = True
+            for layer in runner.model.model.layers:
+                layer.self_attn.fused = True
+        assert c == [x[:4] for x in a], "fused and unfused layer paths differ"
     finally:
         close(llm)
 

@@ -415,8 +415,9 @@ void gemm_dlds_kernel(const GemmParams p) {
   // copy side: byte offset of this lane's piece for each pass, relative to the tile's first row
   // (rows past the end are clamped to the last row; their results are never stored)
   const unsigned char *xbase = p.x + m0 * p.ldx_bytes + static_cast<int64_t>(k_begin) * 2;
-  // int8 weights are in tile order: the row term is part of woff, the K term counts 1 KiB chunks of 32
-  const unsigned char *wbase = W8 ? p.w + static_cast<int64_t>(k_begin / 32) * 1024
+  // int8 weights are in tile order: the tile's first 32-row group and the K term (1 KiB chunks of 32) make the
+  // 64-bit base, woff counts row groups from there (a weight may exceed 2 GiB; a tile never does)
+  const unsigned char *wbase = W8 ? p.w + (static_cast<int64_t>(n0 >> 5) * (p.K / 32) + k_begin / 32) * 1024
                                   : p.w + n0 * ldw_bytes + static_cast<int64_t>(k_begin) * 2;
   unsigned int xoff[XP], woff[WP];
   {
@@ -434,7 +435,7 @@ void gemm_dlds_kernel(const GemmParams p) {
       for (int q = 0; q < WP; ++q) {
         // atom (row n, piece pw of the K-tile) of the tile-ordered weight, relative to the K-tile's first chunk
         const int n = min(n0 + q * (NW * 16) + rw, p.N - 1);
-        woff[q] = static_cast<unsigned int>((n >> 5) * (p.K * 32) + (pw >> 1) * 1024 + (pw & 1) * 512 + (n & 31) * 16);
+        woff[q] = static_cast<unsigned int>(((n - n0) >> 5) * (p.K * 32) + (pw >> 1) * 1024 + (pw & 1) * 512 + (n & 31) * 16);
       }
     } else {
 #pragma unroll
@@ -1185,7 +1186,7 @@ inline const GemmTuning &gemm_tuning() {
       int lo = 0, hi = 0;
       if (sscanf(e, "%d,%d", &lo, &hi) == 2) {
         g.ws_min_m = lo < 1 ? 1 : lo;
-        g.ws_max_m = hi > 256 ? 256 : hi;
+        g.ws_max_m = hi > 224 ? 224 : hi;  // seven token tiles of 32 is the tallest instance
       }
     }
     if (const char *e = getenv("TLF_GEMM_WSTREAM_SPLITS")) g.ws_splits = atoi(e) > 0 ? atoi(e) : 0;
@@ -1300,7 +1301,7 @@ inline bool plan_wstream(int M, int N, int K, int act, GemmPlan &g) {
   // elsewhere one part is 5-15 % faster (gate_up at 32 tokens 19.5 against 20.8 us, qkv 11.2 against 12.0)
   int kg = ktiles % 2 == 0 && kt_per >= 4 && (narrow ? ktiles >= 128 : M > 32) ? 2 : 1;
   if (t.ws_kg && (t.ws_kg == 1 || ktiles % 2 == 0)) kg = t.ws_kg;
-  if (tm > 4 && !(kg == 2 && cols == 3)) return false;  // the tall instances exist in that form only
+  if (tm > 7 || (tm > 4 && !(kg == 2 && cols == 3))) return false;  // the tall instances exist in that form only
   g.stages = tm >= 7 ? 2 : kg == 2 && tm >= 3 ? 3 : 4;
   g.occ = kg;
   g.kgroups = kg;

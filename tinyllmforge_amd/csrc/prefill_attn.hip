@@ -18,12 +18,19 @@
 // two 16-token sub-tiles is exactly the 32-token B operand of the second product:
 // P never leaves registers.
 //
-// The second product runs in fp16 (v_mfma_f32_16x16x32_f16): P lies in [0, 1], where fp16 keeps 11
-// significant bits (a single bf16 P, 8 bits, misses the 1e-3 relative-L2 bar against an exact softmax; a
-// bf16 hi + lo pair meets it at twice the MFMAs and three more vector-ALU operations per score), and V is
-// converted to fp16 once, when its tile is staged: exact for e4m3 rows, exact for bf16 rows between 6.1e-5
-// and 65504 in magnitude (smaller values keep 2^-24 absolute resolution, larger ones saturate at 65504:
-// the conversion rounds toward zero, which never produces an infinity).
+// The second product runs in fp16 (v_mfma_f32_16x16x32_f16): fp16 keeps 11 significant bits of P (a single
+// bf16 P, 8 bits, misses the 1e-3 relative-L2 bar against an exact softmax; a bf16 hi + lo pair meets it at
+// twice the MFMAs and three more vector-ALU operations per score), and V is converted to fp16 once, when its
+// tile is staged (exact for e4m3 rows).  Two guards keep the input domain that of bf16 operands:
+//  - P is carried as 2^15 p (the factor sits in the exponent argument and in the running sum alike, so it
+//    cancels in O / l): weights down to 2^-29 of the row maximum are normal fp16 numbers.  Unscaled, every
+//    weight below 2^-14 would be an fp16 subnormal, and a row with one dominant key and thousands of faint ones
+//    would lose their mass from the numerator but not from the denominator.
+//  - a bf16 V tile that fp16 cannot hold (some |v| >= 65536, or no element as large as 2^-9, where the whole
+//    tile would sit in or near the subnormal range) is staged as it is and multiplied in bf16, with P as a
+//    bf16 hi + lo pair: the choice is made per 64-token tile from a vote of the staging threads.  A tile with
+//    some |v| >= 2^112, where 2^15 p v could leave fp32, ends the 2^15 carry for the rest of the row tile
+//    (accumulators and sums are scaled back once, every later tile is multiplied in bf16).
 #include <stdlib.h>
 
 #include "common.h"
@@ -71,6 +78,12 @@ __device__ __forceinline__ unsigned int pack_f16x2(float lo, float hi) {  // rou
   return __builtin_bit_cast(unsigned int, r);
 }
 constexpr float kPLog2e = 1.4426950408889634f;
+constexpr float kPShift = 15.0f;          // P is carried as 2^15 p
+// bf16 bit patterns (sign cleared) that bound what a tile may hold for the fp16 product
+constexpr unsigned int kVBigBits = 0x4780u;     // 65536: the first bf16 above the largest finite fp16
+constexpr unsigned int kVDecentBits = 0x3b00u;  // 2^-9
+constexpr unsigned int kVHugeBits = 0x7780u;    // 2^112: 2^15 p v may overflow fp32 from here on
+typedef unsigned short ushortx2 __attribute__((ext_vector_type(2)));
 
 struct PrefillParams {
   const unsigned short *q;
@@ -145,7 +158,8 @@ template <int CT, bool KV8, int NWV>
 __global__ __launch_bounds__(64 * NWV) __attribute__((amdgpu_waves_per_eu(2, 2)))  // 256 registers: two waves per SIMD
 void prefill_attn_kernel(const PrefillParams p) {
   __shared__ __attribute__((aligned(16))) unsigned short Ks[kBKV][kPRowK];  // bf16, rows in k_tile_row order
-  __shared__ __attribute__((aligned(16))) unsigned short Vs[kBKV][kPRowV];  // fp16
+  __shared__ __attribute__((aligned(16))) unsigned short Vs[kBKV][kPRowV];  // fp16 (bf16 for a tile fp16 cannot hold)
+  __shared__ __attribute__((aligned(16))) unsigned int vvote[8];            // per wave: what its V slice holds
   // Workgroup -> (sequence, KV head, row tile).  Workgroups go to the 8 XCDs round robin by their linear id, and
   // each XCD has its own L2: when the (sequence, KV head) pairs divide evenly, pair j runs entirely on XCD j % 8,
   // so the K/V rows its row tiles share are fetched into one L2 instead of eight.  An XCD takes its pairs
@@ -252,7 +266,39 @@ void prefill_attn_kernel(const PrefillParams p) {
       }
     }
   };
-  auto store_tile = [&]() __attribute__((always_inline)) {
+  // What this wave's slice of the V tile in vreg holds: bit 0 some |v| >= 65536, bit 1 some |v| >= 2^-9,
+  // bit 2 anything but zeros, bit 3 some |v| >= 2^112.  (e4m3 rows always fit fp16.)
+  auto vote_tile = [&]() __attribute__((always_inline)) {
+    if constexpr (!KV8) {
+      ushortx2 mx = ushortx2{0, 0};
+#pragma unroll
+      for (int i = 0; i < kPasses; ++i) {
+        const unsigned int w[4] = {vreg[i].x, vreg[i].y, vreg[i].z, vreg[i].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          mx = __builtin_elementwise_max(mx, __builtin_bit_cast(ushortx2, w[e] & 0x7fff7fffu));
+      }
+      const unsigned int m = mx[0] > mx[1] ? mx[0] : mx[1];
+      const unsigned int bits = (__builtin_amdgcn_ballot_w64(m >= kVBigBits) ? 1u : 0u) |
+                                (__builtin_amdgcn_ballot_w64(m >= kVDecentBits) ? 2u : 0u) |
+                                (__builtin_amdgcn_ballot_w64(m != 0u) ? 4u : 0u) |
+                                (__builtin_amdgcn_ballot_w64(m >= kVHugeBits) ? 8u : 0u);
+      if (lane == 0) vvote[wave] = bits;
+    }
+  };
+  // After the barrier that follows vote_tile(): the OR of the waves' votes (workgroup uniform)
+  auto tile_votes = [&]() __attribute__((always_inline)) -> unsigned int {
+    if constexpr (KV8) return 0u;
+    unsigned int any = 0;
+#pragma unroll
+    for (int w = 0; w < NWV; w += 4) {
+      const uint4 t = *reinterpret_cast<const uint4 *>(&vvote[w]);
+      any |= t.x | t.y | t.z | t.w;
+    }
+    return __builtin_amdgcn_readfirstlane(any);
+  };
+  auto votes_need_bf16 = [](unsigned int any) { return (any & 1u) || ((any & 6u) == 4u); };
+  auto store_tile = [&](bool v_as_bf16) __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < kPasses; ++i) {
       const int t = i * kRowsPerPass + trow;
@@ -268,9 +314,12 @@ void prefill_attn_kernel(const PrefillParams p) {
         *reinterpret_cast<uint4 *>(&Vs[t][64 + ch * 8]) = hi;
       } else {
         *reinterpret_cast<uint4 *>(&Ks[kr][ch * 8]) = kreg[i];
-        *reinterpret_cast<uint4 *>(&Vs[t][ch * 8]) =
-            make_uint4(bf16x2_to_f16x2(vreg[i].x), bf16x2_to_f16x2(vreg[i].y), bf16x2_to_f16x2(vreg[i].z),
-                       bf16x2_to_f16x2(vreg[i].w));
+        if (v_as_bf16)
+          *reinterpret_cast<uint4 *>(&Vs[t][ch * 8]) = vreg[i];
+        else
+          *reinterpret_cast<uint4 *>(&Vs[t][ch * 8]) =
+              make_uint4(bf16x2_to_f16x2(vreg[i].x), bf16x2_to_f16x2(vreg[i].y), bf16x2_to_f16x2(vreg[i].z),
+                         bf16x2_to_f16x2(vreg[i].w));
       }
     }
   };
@@ -286,11 +335,27 @@ void prefill_attn_kernel(const PrefillParams p) {
   }
 
   load_tile(0);
-  store_tile();
+  vote_tile();
+  lds_barrier();
+  unsigned int votes = tile_votes();
+  float pshift = kPShift;            // P is carried as 2^pshift p: 15, or 0 once a tile with huge values was met
+  bool v_bf16 = votes_need_bf16(votes);   // of the tile in LDS
+  bool v_huge = (votes & 8u) != 0;
+  store_tile(v_bf16);
   lds_barrier();
   for (int kv0 = 0; kv0 < kv_end; kv0 += kBKV) {
     const bool more = kv0 + kBKV < kv_end;
     if (more) load_tile(kv0 + kBKV);
+    if (!KV8 && v_huge && pshift != 0.f) {  // workgroup uniform, at most once per workgroup
+      const float back = 0x1p-15f;
+#pragma unroll
+      for (int c = 0; c < CT; ++c) {
+        l_run[c] *= back;
+        rescale16(acc[c], 0, back);
+        rescale16(acc[c], 4, back);
+      }
+      pshift = 0.f;
+    }
     // tiles that end at or before the first row's limit and inside lk need no mask
     const bool need_mask = (kv0 + kBKV - 1 > shift + row0) || (kv0 + kBKV > lk);
 #pragma unroll
@@ -316,7 +381,7 @@ void prefill_attn_kernel(const PrefillParams p) {
         }
       }
       // lane (n, g) of column tile c holds tokens kv0 + hh*32 + g*8 + j, j = 0..7
-      f16x8 ph[CT];
+      uint4 ph[CT], pl[CT];  // fp16 P; or bf16 P as a hi + lo pair for a tile multiplied in bf16
 #pragma unroll
       for (int c = 0; c < CT; ++c) {
         // (the softmax is where this kernel's vector-ALU time goes: raw v_exp_f32, one fused
@@ -343,12 +408,24 @@ void prefill_attn_kernel(const PrefillParams p) {
         const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
         const float alpha = __builtin_amdgcn_exp2f(m_run[c] - m_use);
         float pv[8];
+        const float shift_m = pshift - m_use;
 #pragma unroll
-        for (int j = 0; j < 8; ++j)  // p = 2^(s * scale - m): arguments are <= 0, a flushed denormal result is an exact 0 weight
-          pv[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[j], scale_log2, -m_use));
+        for (int j = 0; j < 8; ++j)  // 2^15 p = 2^(s * scale - m + 15): at most 2^15; a flushed denormal result is an exact 0 weight
+          pv[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[j], scale_log2, shift_m));
         const float psum = ((pv[0] + pv[1]) + (pv[2] + pv[3])) + ((pv[4] + pv[5]) + (pv[6] + pv[7]));
-        ph[c] = __builtin_bit_cast(f16x8, make_uint4(pack_f16x2(pv[0], pv[1]), pack_f16x2(pv[2], pv[3]),
-                                                     pack_f16x2(pv[4], pv[5]), pack_f16x2(pv[6], pv[7])));
+        if (!KV8 && v_bf16) {  // workgroup uniform
+          unsigned int hi[4], lo[4];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            hi[j] = pack_bf16x2(pv[2 * j], pv[2 * j + 1]);
+            lo[j] = pack_bf16x2(pv[2 * j] - __uint_as_float(hi[j] << 16), pv[2 * j + 1] - __uint_as_float(hi[j] & 0xffff0000u));
+          }
+          ph[c] = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+          pl[c] = make_uint4(lo[0], lo[1], lo[2], lo[3]);
+        } else {
+          ph[c] = make_uint4(pack_f16x2(pv[0], pv[1]), pack_f16x2(pv[2], pv[3]), pack_f16x2(pv[4], pv[5]),
+                             pack_f16x2(pv[6], pv[7]));
+        }
         l_run[c] = l_run[c] * alpha + psum;
         m_run[c] = m_new;
         // Rescale of the accumulators, skipped (wave-uniform branch) while no lane's running max moved, which is
@@ -364,16 +441,30 @@ void prefill_attn_kernel(const PrefillParams p) {
       for (int d = 0; d < 8; ++d) {
         const shortx4 v0 = lds_read_tr16(&Vs[vt][d * 16 + (n & 3) * 4]);
         const shortx4 v1 = lds_read_tr16(&Vs[vt + 4][d * 16 + (n & 3) * 4]);
-        const f16x8 vf = __builtin_bit_cast(
-            f16x8, make_uint4(__builtin_bit_cast(uint2, v0).x, __builtin_bit_cast(uint2, v0).y,
-                              __builtin_bit_cast(uint2, v1).x, __builtin_bit_cast(uint2, v1).y));
+        const uint4 vraw = make_uint4(__builtin_bit_cast(uint2, v0).x, __builtin_bit_cast(uint2, v0).y,
+                                      __builtin_bit_cast(uint2, v1).x, __builtin_bit_cast(uint2, v1).y);
+        if (!KV8 && v_bf16) {
+          const bf16x8 vb = __builtin_bit_cast(bf16x8, vraw);
 #pragma unroll
-        for (int c = 0; c < CT; ++c) acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, ph[c], acc[c][d], 0, 0, 0);
+          for (int c = 0; c < CT; ++c) {
+            acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vb, __builtin_bit_cast(bf16x8, ph[c]), acc[c][d], 0, 0, 0);
+            acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vb, __builtin_bit_cast(bf16x8, pl[c]), acc[c][d], 0, 0, 0);
+          }
+        } else {
+          const f16x8 vf = __builtin_bit_cast(f16x8, vraw);
+#pragma unroll
+          for (int c = 0; c < CT; ++c)
+            acc[c][d] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, __builtin_bit_cast(f16x8, ph[c]), acc[c][d], 0, 0, 0);
+        }
       }
     }
+    if (more) vote_tile();   // of the tile that was loaded while this one was multiplied
     lds_barrier();
     if (more) {
-      store_tile();
+      votes = tile_votes();
+      v_huge = (votes & 8u) != 0;
+      v_bf16 = votes_need_bf16(votes) || v_huge || pshift == 0.f;
+      store_tile(v_bf16);
       lds_barrier();
     }
   }

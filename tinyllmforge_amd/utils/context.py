@@ -8,7 +8,7 @@ nothing is allocated for that), so a caller must not hold on to ``get_context()`
 """
 from __future__ import annotations
 
-# field -> value after reset_context(); the order is the positional order of set_context()
+# field -> value after reset_context(), in the positional order of set_context()
 _FIELDS = (
     ("is_prefill", False),      # prefill or decode step
     ("cu_seqlens_q", None),     # prefill: int32 [B + 1] prefix sums of the query lengths
@@ -42,19 +42,15 @@ def get_context() -> Context:
     return _CURRENT
 
 
-def set_context(is_prefill, *values, **named):
-    """``set_context(is_prefill, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, slot_mapping,
-    context_lens, block_tables)``, every argument after the first optional, positional or by name."""
-    _CURRENT.clear()
-    _CURRENT.is_prefill = is_prefill
-    if len(values) > len(_FIELDS) - 1:
-        raise TypeError(f"set_context takes at most {len(_FIELDS)} positional arguments")
-    for (name, _), value in zip(_FIELDS[1:], values):
-        setattr(_CURRENT, name, value)
-    for name, value in named.items():
-        if name not in Context.__slots__ or name == "is_prefill":
-            raise TypeError(f"set_context got an unexpected argument {name!r}")
-        setattr(_CURRENT, name, value)
+def set_context(is_prefill, cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=0, max_seqlen_k=0, slot_mapping=None,
+                context_lens=None, block_tables=None):
+    """Publish one step's metadata; every argument after the first is optional, positional or by name
+    (same parameter list as tinyvllm/utils/context.py:21)."""
+    c = _CURRENT
+    c.is_prefill = is_prefill
+    c.cu_seqlens_q, c.cu_seqlens_k = cu_seqlens_q, cu_seqlens_k
+    c.max_seqlen_q, c.max_seqlen_k = max_seqlen_q, max_seqlen_k
+    c.slot_mapping, c.context_lens, c.block_tables = slot_mapping, context_lens, block_tables
 
 
 def reset_context():
