@@ -52,11 +52,17 @@ def parse():
     ap.add_argument("--steps", type=int, default=0,
                     help="engine steps that steps/ms_per_step describe (0 = all); value is always the whole job")
     ap.add_argument("--warmup", type=int, default=1, help="warm-up generate() calls before the timed run")
-    ap.add_argument("--workload", default="e2e", choices=["e2e", "decode_attn", "gemm", "prefill_attn", "c5", "all"])
+    ap.add_argument("--workload", default="e2e",
+                    choices=["e2e", "decode_attn", "gemm", "prefill_attn", "elementwise", "c5", "all"])
     ap.add_argument("--attn-steps", type=int, default=200, help="timed launches of the decode-attention microbench")
     ap.add_argument("--num-seqs", type=int, default=256)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--fp8", action="store_true", help="decode_attn: e4m3 cache rows (BASELINE.json configs[4]'s attention)")
+    ap.add_argument("--hq", type=int, default=32, help="decode_attn: query heads (8 KV heads)")
+    ap.add_argument("--gemm-shapes", default="8b", choices=["8b", "32b", "0.6b", "all"],
+                    help="gemm: projection shapes of which model (configs[2] is 8b)")
+    ap.add_argument("--gemm-m", default="", help="gemm: comma-separated token counts instead of the default list")
     ap.add_argument("--skip-bf16", action="store_true", help="e2e: skip the second run with bf16 linears (profiling)")
     ap.add_argument("--skip-c5", action="store_true", help="e2e: skip the Qwen3-32B-shape run (configs[4])")
     ap.add_argument("--skip-gemm", action="store_true", help="e2e: skip the W8A16 GEMM table (configs[2])")
@@ -161,8 +167,32 @@ def bench_probes(args):
     st = torch.cuda.current_stream().cuda_stream
     tr = time_launches(lambda: _lib.check(lib.tlf_probe_read(src.data_ptr(), n, sink.data_ptr(), st), "probe"), 30, 5)
     tc = time_launches(lambda: _lib.check(lib.tlf_probe_copy(src.data_ptr(), dst.data_ptr(), n, st), "probe"), 30, 5)
-    return dict(read_GBps=round(n / (tr["mean_ms"] * 1e-3) / 1e9, 1),
-                copy_GBps=round(2 * n / (tc["mean_ms"] * 1e-3) / 1e9, 1), bytes=n)
+    res = dict(read_GBps=round(n / (tr["mean_ms"] * 1e-3) / 1e9, 1),
+               copy_GBps=round(2 * n / (tc["mean_ms"] * 1e-3) / 1e9, 1), bytes=n)
+    # what the matrix cores sustain from registers, on small-integer and on random operands
+    out = torch.empty(512 * 256, dtype=torch.float32, device="cuda")
+    iters = 4000
+    flop = 2.0 * 32 * 32 * 16 * 16 * iters * 2048
+    mf = {}
+    for mode, name in ((0, "small_int_TFLOPs"), (1, "random_TFLOPs")):
+        t = time_launches(lambda: _lib.check(lib.tlf_probe_mfma(out.data_ptr(), iters, mode, st), "probe"), 5, 2)
+        mf[name] = round(flop / (t["mean_ms"] * 1e-3) / 1e12, 1)
+    mf["note"] = "register-only v_mfma_f32_32x32x16_bf16 stream, two waves per SIMD: the clock drops on random data"
+    res["mfma_probe"] = mf
+    # an HBM stream and an L2-resident stream through the same CUs at once: the launch takes the sum of the two
+    small = src[:1 << 20]
+    def mix(big_bytes, eighths):
+        t = time_launches(lambda: _lib.check(lib.tlf_probe_mix(src.data_ptr(), big_bytes, small.data_ptr(), 1 << 20, eighths,
+                                                               sink.data_ptr(), st), "probe"), 10, 3)
+        return t["mean_ms"] * 1e3
+    hbm_alone = mix(n, 0)
+    both = mix(n, 22)                               # 2.75 KiB out of L2 per KiB from HBM: a GEMM at 128 tokens
+    l2_alone = mix(16 << 20, 22 * 64)               # the same L2 bytes beside a negligible HBM part
+    res["mixed_traffic_probe"] = dict(hbm_1GiB_alone_us=round(hbm_alone, 1), l2_2p75GiB_alone_us=round(l2_alone, 1),
+                                      both_at_once_us=round(both, 1), sum_us=round(hbm_alone + l2_alone, 1),
+                                      note="4 waves per CU stream from HBM, 4 re-read 1 MiB out of L2; loads return in "
+                                           "order through a CU's L1, so the two do not overlap")
+    return res
 
 
 def bench_decode_attn(args, fp8=False, hq=32):
@@ -218,9 +248,13 @@ def cpu_baseline_decode(case, budget_s=20.0):
 
 # ----------------------------------------------------------------------------- config 3
 GEMM_SHAPES = {"qkv": (6144, 4096), "o_proj": (4096, 4096), "gate_up": (24576, 4096), "down": (4096, 12288)}
+GEMM_SHAPES_32B = {"qkv_32b": (10240, 5120), "o_proj_32b": (5120, 8192), "gate_up_32b": (51200, 5120),
+                   "down_32b": (5120, 25600)}
+GEMM_SHAPES_06B = {"qkv_0.6b": (4096, 1024), "o_proj_0.6b": (1024, 2048), "gate_up_0.6b": (6144, 1024),
+                   "down_0.6b": (1024, 3072)}
 
 
-def bench_gemm(args, ms=(1, 16, 64, 128, 256, 2048, 8192)):
+def bench_gemm(args, ms=(1, 16, 64, 128, 256, 2048, 8192), shapes=None):
     """W8A16 GEMM table.  Up to M = 256 a decode step finds its weights in HBM (a layer's weights were last
     touched one whole step ago), so those cells cycle through enough copies of the weight to exceed the
     256 MB Infinity Cache several times ("cold"); the same call on one resident copy is reported beside it
@@ -228,8 +262,13 @@ def bench_gemm(args, ms=(1, 16, 64, 128, 256, 2048, 8192)):
     import torch
     from tinyllmforge_amd import ops as P
     torch.manual_seed(0)
+    import ctypes
+    from tinyllmforge_amd import _lib
+    lib = _lib.load()
     rows = []
-    for name, (N, K) in GEMM_SHAPES.items():
+    if getattr(args, "gemm_m", ""):
+        ms = tuple(int(a) for a in args.gemm_m.split(","))
+    for name, (N, K) in (shapes or GEMM_SHAPES).items():
         copies = max(2, -(-(768 << 20) // (N * K)))
         wqs = [P.pack_w8(torch.randint(-127, 128, (N, K), device="cuda", dtype=torch.int8)) for _ in range(copies)]
         scale = torch.rand(N, device="cuda") * 9e-3 + 1e-3
@@ -245,7 +284,10 @@ def bench_gemm(args, ms=(1, 16, 64, 128, 256, 2048, 8192)):
             nbytes = N * K + 4 * N + 2 * M * K + 2 * M * N
             flops = 2.0 * M * N * K
             bound = "hbm" if M <= 128 else "mfma"
-            rows.append(dict(shape=name, M=M, N=N, K=K, us=round(sec * 1e6, 2), weights="cold" if M <= 256 else "warm",
+            plan = (ctypes.c_int32 * 8)()
+            lib.tlf_gemm_plan(M, N, K, 1, plan)
+            rows.append(dict(shape=name, M=M, N=N, K=K, plan=list(plan)[:6],
+                             us=round(sec * 1e6, 2), weights="cold" if M <= 256 else "warm",
                              us_warm=round(warm * 1e6, 2), GBps=round(nbytes / sec / 1e9, 1),
                              TFLOPs=round(flops / sec / 1e12, 1), bound=bound,
                              frac=round((nbytes / sec / 1e9 / HBM_PEAK_GBPS) if bound == "hbm"
@@ -279,6 +321,101 @@ def cpu_baseline_gemm(budget_s=20.0):
     return dict(value=round(flops / spent / 1e12, 4), unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
                 sample=f"qkv projection (N={N}, K={K}) at M = {sorted(set(done))}, {len(done)} calls, "
                        f"{spent:.1f} s of CPU oracle time")
+
+
+# ----------------------------------------------------------------------------- elementwise kernels
+def bench_elementwise(args, sizes=(16384, 256)):
+    """The single-pass kernels at the 8B widths (hidden 4096, 32 / 8 heads of 128, intermediate 12288, vocabulary
+    151,936) at a prefill step's size (16,384 tokens) and a decode step's (256): algorithmic bytes (every input
+    element read once, every output element written once) over the hipGraph-timed launch, against 8 TB/s.
+    At 16,384 tokens each kernel cycles through enough independent copies of its tensors to exceed the 256 MB
+    Infinity Cache ("cold"); at 256 tokens the tensors are a few MB and sit in L2, as they do between two kernels
+    of a decode step ("warm": these cells measure launch and latency, not bandwidth)."""
+    import torch
+    from tinyllmforge_amd import ops as P
+    from tinyllmforge_amd.layers.rotary_embedding import build_cos_sin_cache
+    torch.manual_seed(0)
+    BF, dev = torch.bfloat16, "cuda"
+    H, Hq, Hkv, Dh, I, V = 4096, 32, 8, 128, 12288, 151936
+    QKV = (Hq + 2 * Hkv) * Dh
+    tab = build_cos_sin_cache(Dh, 40960, 1e6).to(dev)
+    w_h = torch.ones(H, dtype=BF, device=dev)
+    w_d = torch.ones(Dh, dtype=BF, device=dev)
+    emb = (torch.randn(V, H, device=dev) * 0.02).to(BF)
+    rows = []
+
+    def timed(name, n, nbytes, per_copy_bytes, make, cold=None):
+        cold = n > 1024 if cold is None else cold
+        copies = max(2, -(-(768 << 20) // max(1, per_copy_bytes))) if cold else 1
+        calls = [make() for _ in range(copies)]
+
+        def cycle():
+            for c in calls:
+                c()
+        sec = time_graph(cycle, launches=40 if copies == 1 else 2, replays=10) * 1e-3 / copies
+        gbps = nbytes / sec / 1e9
+        rows.append(dict(kernel=name, tokens=n, us=round(sec * 1e6, 2), algorithmic_MB=round(nbytes / 1e6, 2),
+                         GBps=round(gbps, 1), frac=round(gbps / HBM_PEAK_GBPS, 4), data="cold" if copies > 1 else "warm"))
+        del calls
+        torch.cuda.empty_cache()
+
+    for n in sizes:
+        nblk = -(-n // 256) + 1
+
+        def mk_store():
+            qkv = torch.randn(n, QKV, device=dev).to(BF)
+            key = torch.randn(n, Hkv, Dh, device=dev).to(BF)
+            val = qkv[:, (Hq + Hkv) * Dh:].view(n, Hkv, Dh)          # a view into the projection, as the model passes it
+            kc = torch.zeros(nblk, 256, Hkv, Dh, dtype=BF, device=dev)
+            vc = torch.zeros_like(kc)
+            slots = torch.randperm(nblk * 256, device=dev)[:n].to(torch.int32)
+            return lambda: P.store_kvcache(key, val, kc, vc, slots)
+        timed("store_kvcache", n, n * (4 * Hkv * Dh * 2 + 4), n * (QKV * 2 + 3 * Hkv * Dh * 2), mk_store)
+
+        def mk_rms():
+            x = torch.randn(n, H, device=dev).to(BF)
+            return lambda: P.rms_norm(x, w_h, 1e-6)
+        timed("rmsnorm", n, n * H * 4, n * H * 4, mk_rms)
+
+        def mk_add_rms():
+            x = torch.randn(n, H, device=dev).to(BF)
+            r = torch.randn(n, H, device=dev).to(BF)
+            return lambda: P.add_rms_norm(x, r, w_h, 1e-6)
+        timed("add_rmsnorm", n, n * H * 8, n * H * 8, mk_add_rms)
+
+        def mk_rope():
+            q = torch.randn(n, Hq * Dh, device=dev).to(BF)
+            k = torch.randn(n, Hkv * Dh, device=dev).to(BF)
+            pos = torch.randint(0, 4096, (n,), device=dev)
+            return lambda: P.rope(pos, q, k, tab, Dh)
+        timed("rope", n, n * ((Hq + Hkv) * Dh * 4 + 8 + Dh * 4), n * (Hq + Hkv) * Dh * 4, mk_rope)
+
+        def mk_fused():
+            qkv = torch.randn(n, QKV, device=dev).to(BF)
+            pos = torch.randint(0, 4096, (n,), device=dev)
+            kc = torch.zeros(nblk, 256, Hkv, Dh, dtype=BF, device=dev)
+            vc = torch.zeros_like(kc)
+            slots = torch.randperm(nblk * 256, device=dev)[:n].to(torch.int32)
+            return lambda: P.qknorm_rope_store(qkv, w_d, w_d, 1e-6, pos, tab, Hq, Hkv, Dh, kc, vc, slots)
+        timed("qknorm_rope_store", n, n * (QKV * 2 + Hq * Dh * 2 + 2 * Hkv * Dh * 2 + 8 + Dh * 4 + 4),
+              n * (QKV * 2 + Hq * Dh * 2 + 2 * Hkv * Dh * 2), mk_fused)
+
+        def mk_silu():
+            x = torch.randn(n, 2 * I, device=dev).to(BF)
+            return lambda: P.silu_and_mul(x)
+        timed("silu_and_mul", n, n * I * 6, n * I * 6, mk_silu)
+
+        def mk_emb():
+            ids = torch.randint(0, V, (n,), device=dev)
+            return lambda: P.embedding(ids, emb)
+        timed("embedding", n, n * (H * 4 + 8), n * H * 4, mk_emb)
+
+    def mk_argmax():
+        logits = torch.randn(256, V, device=dev).to(BF)
+        return lambda: P.argmax(logits)
+    # 78 MB of logits a copy: ten copies exceed the Infinity Cache three times
+    timed("argmax (256 x 151936)", 256, 256 * V * 2 + 256 * 8, 256 * V * 2, mk_argmax, cold=True)
+    return rows
 
 
 # ----------------------------------------------------------------------------- prefill attention microbench
@@ -489,12 +626,14 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
     extra = {}
-    attn = bench_decode_attn(args)
+    attn = bench_decode_attn(args, fp8=args.fp8, hq=args.hq) if args.workload == "decode_attn" else bench_decode_attn(args)
     roofline = attn["roofline"]
     extra["paged_decode_GBps_back_to_back"] = round(attn["value"], 1)
     extra["hbm_probe"] = bench_probes(args)
     if args.workload in ("gemm", "all"):
-        extra["w8a16_gemm"] = bench_gemm(args)
+        sets = {"8b": GEMM_SHAPES, "32b": GEMM_SHAPES_32B, "0.6b": GEMM_SHAPES_06B,
+                "all": {**GEMM_SHAPES, **GEMM_SHAPES_32B, **GEMM_SHAPES_06B}}
+        extra["w8a16_gemm"] = bench_gemm(args, shapes=sets[args.gemm_shapes])
     if args.workload == "gemm":   # its own line: the linear-layer microbench (BASELINE.json configs[2])
         best = max(r["TFLOPs"] for r in extra["w8a16_gemm"])
         print(json.dumps({
@@ -505,6 +644,20 @@ def main():
                                    "Qwen3-8B projection shapes, M = 1 ... 8192, random normal x, random int8 W"},
             "roofline": roofline, "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline_gemm(),
             "extra": extra}))
+        return
+    if args.workload == "elementwise":   # its own line: the single-pass kernels
+        rows = bench_elementwise(args)
+        extra["elementwise"] = rows
+        big = [r for r in rows if r["data"] == "cold"]
+        worst = min(big, key=lambda r: r["frac"])
+        print(json.dumps({
+            "metric": "elementwise kernels: algorithmic GB/s vs HBM peak (worst kernel at 16,384 tokens)", "value": worst["GBps"],
+            "unit": "GB/s", "n_gpus": 1, "steps": 20, "warmup": 1, "ms_per_step": round(worst["us"] * 1e-3, 5),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "single-pass kernels at the Qwen3-8B widths, 16,384 and 256 tokens: " + worst["kernel"]},
+            "roofline": {"bound": "hbm", "achieved": worst["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                         "frac": worst["frac"], "traffic": None, "kernel": worst["kernel"]},
+            "cpu_baseline": None, "extra": extra}))
         return
     if args.workload == "prefill_attn":   # its own line: the prefill-attention microbench
         rows = bench_prefill_attn(args)
@@ -525,8 +678,9 @@ def main():
             "metric": "paged-decode HBM GB/s vs peak", "value": round(attn["value"], 1), "unit": "GB/s", "n_gpus": 1,
             "steps": args.attn_steps, "warmup": 30, "ms_per_step": round(attn["ms_per_step"], 5),
             "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-            "config": {"workload": "BASELINE.json configs[1]: paged decode attention microbench, B=%d Hq=32 Hkv=8 "
-                                   "Dh=128 block_size=256 ctx~U[512,4096] pool=2048 blocks" % args.batch,
+            "config": {"workload": "BASELINE.json configs[1]: paged decode attention microbench, B=%d Hq=%d Hkv=8 "
+                                   "Dh=128 block_size=256 ctx~U[512,4096] pool=2048 blocks, %s cache rows"
+                                   % (args.batch, args.hq, "e4m3" if args.fp8 else "bf16"),
                        "total_context_tokens": attn["case"]["total_tokens"]},
             "roofline": roofline, "cpu_baseline": cpu, "extra": extra}
         print(json.dumps(out))
@@ -535,6 +689,7 @@ def main():
     torch.cuda.empty_cache()
     if args.workload == "e2e" and not args.skip_gemm:
         extra["w8a16_gemm"] = bench_gemm(args)          # BASELINE.json configs[2]
+        extra["elementwise"] = bench_elementwise(args)
     # the decode microbench on e4m3 rows with 64 query heads (the 32B shape's attention)
     a8 = bench_decode_attn(args, fp8=True, hq=64)
     a8.pop("case")

@@ -62,6 +62,8 @@ SIGNATURES = {
     "tlf_embedding": (c_int32, [_P, _P, _P, _I32, _I32, _I32, _P]),
     "tlf_probe_read": (c_int32, [_P, _SZ, _P, _P]),
     "tlf_probe_copy": (c_int32, [_P, _P, _SZ, _P]),
+    "tlf_probe_mfma": (c_int32, [_P, c_int32, c_int32, _P]),
+    "tlf_probe_mix": (c_int32, [_P, _SZ, _P, _SZ, c_int32, _P, _P]),
 }
 
 

@@ -65,7 +65,100 @@ __global__ __launch_bounds__(256) void probe_copy_kernel(const uint4 *__restrict
     dst[i] = src[i];
 }
 
+// Register-only MFMA stream: what the matrix cores sustain with nothing to wait for.  Every wave issues
+// 16 * iters v_mfma_f32_32x32x16_bf16 on four independent accumulators from operands that never change:
+// small integers (mode 0) or pseudo-random bf16 activations times int8-valued weights (mode 1).  The two
+// differ on this part: the clock drops under the switching activity of random data.
+__global__ __launch_bounds__(256) void probe_mfma_kernel(float *__restrict__ out, int iters, int mode) {
+  bf16x8 a, b;
+  unsigned int h = threadIdx.x * 2654435761u + blockIdx.x * 40503u + 17u;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    h = h * 1664525u + 1013904223u;
+    const float fa = mode ? (static_cast<int>(h >> 8) % 2001 - 1000) * 1e-3f : static_cast<float>((threadIdx.x + i) & 3);
+    h = h * 1664525u + 1013904223u;
+    const float fb = mode ? static_cast<float>(static_cast<int>(h >> 8) % 255 - 127) : static_cast<float>(i & 1);
+    a[i] = static_cast<__bf16>(fa);
+    b[i] = static_cast<__bf16>(fb);
+  }
+  floatx16 acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[j], 0, 0, 0);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s += acc[j][v];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+// Two streams through one CU's vector-memory path at once: waves 0 .. 3 of every workgroup read a region of
+// their own once (from HBM), waves 4 .. 7 re-read a small region that stays in L2, l2_units KiB for every KiB
+// of the first kind.  Measured on MI355X the launch takes the SUM of the times the two streams take alone
+// (loads return in order through a CU's L1, so an L2 hit queues behind the HBM misses issued before it):
+// a decode-size GEMM, whose workgroups all re-read the activations out of L2 while they stream their weights
+// from HBM, pays for both in full.
+__global__ __launch_bounds__(512) void probe_mix_kernel(const unsigned char *__restrict__ big, size_t kib_per_wave,
+                                                        const unsigned char *__restrict__ small_, size_t small_kib,
+                                                        int l2_eighths, unsigned int *__restrict__ sink) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  unsigned int acc = 0;
+  uint4 v[16];
+  if (wave < 4) {
+    const unsigned char *p = big + (static_cast<size_t>(blockIdx.x) * 4 + wave) * kib_per_wave * 1024 + lane * 16;
+    for (size_t i = 0; i + 16 <= kib_per_wave; i += 16) {
+#pragma unroll
+      for (int d = 0; d < 16; ++d) v[d] = load_nt_u4(p + (i + d) * 1024);
+#pragma unroll
+      for (int d = 0; d < 16; ++d) acc ^= v[d].x ^ v[d].w;
+    }
+  } else {
+    const size_t n = kib_per_wave * l2_eighths / 8;
+    size_t c = (static_cast<size_t>(wave) * 37 + blockIdx.x * 11) % small_kib;
+    for (size_t i = 0; i + 16 <= n; i += 16) {
+#pragma unroll
+      for (int d = 0; d < 16; ++d) {
+        v[d] = *reinterpret_cast<const uint4 *>(small_ + c * 1024 + lane * 16);
+        c = c + 1 == small_kib ? 0 : c + 1;
+      }
+#pragma unroll
+      for (int d = 0; d < 16; ++d) acc ^= v[d].x ^ v[d].w;
+    }
+  }
+  if (acc == 0x9e3779b9u && threadIdx.x == 1023) *sink = acc;  // keeps the loads alive, never taken
+}
+
 }  // namespace tlf
+
+extern "C" int tlf_probe_mfma(void *out, int32_t iters, int32_t mode, void *stream) {
+  if (!out) return TLF_E_NULL;
+  if (iters < 0 || (mode != 0 && mode != 1)) return TLF_E_SHAPE;
+  // one workgroup of four waves per CU slot, twice the CUs: two waves per SIMD keep the pipe full
+  hipLaunchKernelGGL(tlf::probe_mfma_kernel, dim3(512), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     static_cast<float *>(out), iters, mode);
+  return tlf::launch_status();
+}
+
+extern "C" int tlf_probe_mix(const void *big, size_t big_bytes, const void *small_region, size_t small_bytes,
+                             int32_t l2_eighths, void *sink, void *stream) {
+  if (!big || !small_region || !sink) return TLF_E_NULL;
+  if (!tlf::aligned16(big) || !tlf::aligned16(small_region)) return TLF_E_ALIGN;
+  const size_t kib_per_wave = big_bytes / 1024 / (256 * 4) / 16 * 16;
+  if (kib_per_wave == 0 || small_bytes < 16 * 1024 || small_bytes % 1024 || l2_eighths < 0) return TLF_E_SHAPE;
+  hipLaunchKernelGGL(tlf::probe_mix_kernel, dim3(256), dim3(512), 0, static_cast<hipStream_t>(stream),
+                     static_cast<const unsigned char *>(big), kib_per_wave,
+                     static_cast<const unsigned char *>(small_region), small_bytes / 1024, l2_eighths,
+                     static_cast<unsigned int *>(sink));
+  return tlf::launch_status();
+}
 
 extern "C" int tlf_probe_read(const void *src, size_t bytes, void *sink, void *stream) {
   if (!src || !sink) return TLF_E_NULL;
