@@ -359,8 +359,17 @@ def bench_elementwise(args, sizes=(16384, 256)):
         del calls
         torch.cuda.empty_cache()
 
+    def slots_of(n, nblk):
+        """Cache slots as the engine hands them out: a prefill step's tokens fill whole 256-token blocks in
+        order, the blocks lie anywhere in the pool; a decode step's tokens are one per sequence, anywhere."""
+        if n <= 1024:
+            return torch.randperm(nblk * 256, device=dev)[:n].to(torch.int32)
+        blocks = torch.randperm(nblk, device=dev)
+        t = torch.arange(n, device=dev)
+        return (blocks[t // 256] * 256 + t % 256).to(torch.int32)
+
     for n in sizes:
-        nblk = -(-n // 256) + 1
+        nblk = -(-n // 256) + 1 if n > 1024 else 2048
 
         def mk_store():
             qkv = torch.randn(n, QKV, device=dev).to(BF)
@@ -368,7 +377,7 @@ def bench_elementwise(args, sizes=(16384, 256)):
             val = qkv[:, (Hq + Hkv) * Dh:].view(n, Hkv, Dh)          # a view into the projection, as the model passes it
             kc = torch.zeros(nblk, 256, Hkv, Dh, dtype=BF, device=dev)
             vc = torch.zeros_like(kc)
-            slots = torch.randperm(nblk * 256, device=dev)[:n].to(torch.int32)
+            slots = slots_of(n, nblk)
             return lambda: P.store_kvcache(key, val, kc, vc, slots)
         timed("store_kvcache", n, n * (4 * Hkv * Dh * 2 + 4), n * (QKV * 2 + 3 * Hkv * Dh * 2), mk_store)
 
@@ -395,7 +404,7 @@ def bench_elementwise(args, sizes=(16384, 256)):
             pos = torch.randint(0, 4096, (n,), device=dev)
             kc = torch.zeros(nblk, 256, Hkv, Dh, dtype=BF, device=dev)
             vc = torch.zeros_like(kc)
-            slots = torch.randperm(nblk * 256, device=dev)[:n].to(torch.int32)
+            slots = slots_of(n, nblk)
             return lambda: P.qknorm_rope_store(qkv, w_d, w_d, 1e-6, pos, tab, Hq, Hkv, Dh, kc, vc, slots)
         timed("qknorm_rope_store", n, n * (QKV * 2 + Hq * Dh * 2 + 2 * Hkv * Dh * 2 + 8 + Dh * 4 + 4),
               n * (QKV * 2 + Hq * Dh * 2 + 2 * Hkv * Dh * 2), mk_fused)

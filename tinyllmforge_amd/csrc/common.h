@@ -37,9 +37,34 @@ __device__ __forceinline__ unsigned short float_to_bf16_bits(float f) {
 
 // SiLU-and-mul with the eager rounding points of the reference (tinyvllm/layers/activation.py:11-14):
 // bf16(silu(g)) * u, the product rounded to bf16 by the caller's pack.  g and u are bf16 values.
+// exp and the division run on the quarter-rate hardware approximations, corrected to about 2 ulp of fp32 in
+// all (the product g * log2(e) keeps its rounding error as a second term, the reciprocal gets one Newton step):
+// with the library expf and an IEEE division the kernel is bound by the vector ALU, not by HBM.  Beyond
+// |g| = 80 the reciprocal's operand nears the end of the fp32 range; those (rare) values take the library path.
 __device__ __forceinline__ float silu_mul_bf16(float g, float u) {
-  const float s = g / (1.0f + expf(-g));
+  float s;
+  if (fabsf(g) <= 80.0f) {
+    const float kL2eHi = 1.44269502162933349609375f, kL2eLo = 1.925963033500011e-08f, kLn2 = 0.693147182464599609375f;
+    const float x = -g;
+    const float hi = __fmul_rn(x, kL2eHi);
+    const float lo = fmaf(x, kL2eLo, fmaf(x, kL2eHi, -hi));    // x * log2(e) - hi
+    const float e0 = __builtin_amdgcn_exp2f(hi);
+    const float d = 1.0f + fmaf(e0, __fmul_rn(lo, kLn2), e0);   // 1 + 2^(hi + lo)
+    float r = __builtin_amdgcn_rcpf(d);
+    r = fmaf(fmaf(-d, r, 1.0f), r, r);
+    s = __fmul_rn(g, r);
+  } else {
+    s = g / (1.0f + expf(-g));
+  }
   return __fmul_rn(bf16_bits_to_float(float_to_bf16_bits(s)), u);
+}
+
+// Value of lane (l - N) mod 16 of the same row of 16 lanes (a DPP move on the vector ALU, no LDS round trip).
+template <int N>
+__device__ __forceinline__ float row_ror(float v) {
+  static_assert(N >= 1 && N <= 15, "rotation inside a row of 16 lanes");
+  const int r = __builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x120 + N, 0xf, 0xf, false);
+  return __int_as_float(r);
 }
 
 __device__ __forceinline__ unsigned int pack_bf16x2(float lo, float hi) {

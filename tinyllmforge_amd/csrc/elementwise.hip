@@ -117,37 +117,70 @@ __global__ __launch_bounds__(256) void rope_kernel(
 
 // --------------------------------------------------------------------------
 // Fused q/k RMSNorm + RoPE + KV-cache store over the qkv projection (qknorm_rope.h): one workgroup handles
-// 16 heads of one token, 16 lanes per head.
+// 16 heads of TOK consecutive tokens, 16 lanes per head.  A lane has the loads of all its TOK pieces in flight
+// before it touches the first (then their table rows, then the arithmetic): with one piece per lane the kernel
+// is bound by the latency of its two dependent loads and by the rate at which 4 KB workgroups can be started.
+template <int TOK>
 __global__ __launch_bounds__(256) void qknorm_rope_store_kernel(const unsigned short *__restrict__ qkv,
-                                                                int64_t qkv_stride, const QkRopeStoreArgs a) {
+                                                                int64_t qkv_stride, int32_t n,
+                                                                const QkRopeStoreArgs a) {
   constexpr int kDh = 128;
-  const int64_t tok = blockIdx.x;
+  const int64_t tok0 = static_cast<int64_t>(blockIdx.x) * TOK;
   const int head = blockIdx.y * 16 + threadIdx.x / 16;
   const int j = threadIdx.x % 16;
   if (head >= a.num_q_heads + 2 * a.num_kv_heads) return;  // whole 16-lane groups leave together
-  const uint4 raw = *reinterpret_cast<const uint4 *>(qkv + tok * qkv_stride + head * kDh + j * 8);
-  qknorm_rope_store_piece(raw, tok, head, j, a);
+  uint4 raw[TOK];
+  QkPieceMeta meta[TOK];
+  QkPieceTable tab[TOK];
+#pragma unroll
+  for (int i = 0; i < TOK; ++i) {
+    const int64_t tok = min(tok0 + i, static_cast<int64_t>(n) - 1);
+    raw[i] = load_nt_u4(qkv + tok * qkv_stride + head * kDh + j * 8);
+    meta[i] = qk_piece_meta(tok, head, a);
+  }
+#pragma unroll
+  for (int i = 0; i < TOK; ++i) tab[i] = qk_piece_table(meta[i], head, j, a);
+#pragma unroll
+  for (int i = 0; i < TOK; ++i)
+    if (tok0 + i < n) qk_piece_finish(raw[i], tok0 + i, head, j, meta[i], tab[i], a);
 }
 
 // --------------------------------------------------------------------------
 // SiLU-and-mul (reference: tinyvllm/layers/activation.py:11-14, eager rounding).
+// A lane handles kSiluUnroll 8-element pieces, 256 lanes apart, and has the loads of all of them in flight
+// before the first exponential.
+constexpr int kSiluUnroll = 4;
 __global__ __launch_bounds__(256) void silu_and_mul_kernel(const unsigned short *__restrict__ x,
                                                            unsigned short *__restrict__ y,
                                                            int64_t rows, int32_t inter) {
   const int cpr = inter / 8;
-  const int64_t item = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  if (item >= rows * cpr) return;
-  const int64_t r = item / cpr;
-  const int c = static_cast<int>(item % cpr);
-  const unsigned short *xr = x + r * 2 * inter;
-  float g[8], u[8], o[8];
-  unpack8(*reinterpret_cast<const uint4 *>(xr + c * 8), g);
-  unpack8(*reinterpret_cast<const uint4 *>(xr + inter + c * 8), u);
+  const int64_t total = rows * cpr;
+  const int64_t item0 = static_cast<int64_t>(blockIdx.x) * (256 * kSiluUnroll) + threadIdx.x;
+  uint4 gp[kSiluUnroll], up[kSiluUnroll];
+  int64_t dst[kSiluUnroll];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    o[i] = silu_mul_bf16(g[i], u[i]);
+  for (int k = 0; k < kSiluUnroll; ++k) {
+    const int64_t item = item0 + k * 256;
+    dst[k] = -1;
+    if (item < total) {
+      const int64_t r = item / cpr;
+      const int c = static_cast<int>(item - r * cpr);
+      const unsigned short *xr = x + r * 2 * inter;
+      gp[k] = load_nt_u4(xr + c * 8);
+      up[k] = load_nt_u4(xr + inter + c * 8);
+      dst[k] = r * inter + c * 8;
+    }
   }
-  *reinterpret_cast<uint4 *>(y + r * inter + c * 8) = pack8(o);
+#pragma unroll
+  for (int k = 0; k < kSiluUnroll; ++k) {
+    if (dst[k] < 0) continue;
+    float g[8], u[8], o[8];
+    unpack8(gp[k], g);
+    unpack8(up[k], u);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = silu_mul_bf16(g[i], u[i]);
+    *reinterpret_cast<uint4 *>(y + dst[k]) = pack8(o);
+  }
 }
 
 // --------------------------------------------------------------------------
@@ -185,15 +218,24 @@ __global__ __launch_bounds__(256) void argmax_partial_kernel(
   const int v0 = chunk * vec_per_chunk;
   const int v1 = min(v0 + vec_per_chunk, nvec);
   unsigned long long best = 0;
-  for (int v = v0 + threadIdx.x; v < v1; v += blockDim.x) {
+  auto take = [&](const uint4 &u, int v) {
     Pack16 p;
-    p.u = *reinterpret_cast<const uint4 *>(lr + static_cast<int64_t>(v) * 8);
+    p.u = u;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
       const unsigned long long key = argmax_key(p.s[i], static_cast<unsigned int>(v * 8 + i));
       best = key > best ? key : best;
     }
+  };
+  int v = v0 + threadIdx.x;
+  for (; v + 3 * 256 < v1; v += 4 * 256) {   // four loads in flight per lane
+    uint4 u[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) u[k] = load_nt_u4(lr + static_cast<int64_t>(v + k * 256) * 8);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) take(u[k], v + k * 256);
   }
+  for (; v < v1; v += 256) take(load_nt_u4(lr + static_cast<int64_t>(v) * 8), v);
   if (chunk == 0) {  // scalar tail when vocab is not a multiple of 8
     const int t = nvec * 8 + threadIdx.x;
     if (t < vocab) {
@@ -335,7 +377,7 @@ int launch_argmax_final(const unsigned long long *keys, int32_t nparts, int64_t 
 }
 
 inline int argmax_chunks(int32_t rows, int32_t vocab) {
-  int by_rows = (1024 + rows - 1) / rows;
+  int by_rows = (2048 + rows - 1) / rows;   // enough workgroups for eight on every CU
   int by_vocab = (vocab + 2047) / 2048;
   int n = by_rows < by_vocab ? by_rows : by_vocab;
   if (n < 1) n = 1;
@@ -418,7 +460,7 @@ int tlf::check_qk_rope_store_args(const void *q_norm_weight, const void *k_norm_
     }
     if (!aligned16(k_cache) || !aligned16(v_cache)) return TLF_E_ALIGN;
   }
-  if (!aligned16(q_out) || !aligned16(q_norm_weight) || !aligned16(k_norm_weight) ||
+  if (!aligned16(q_out) || !aligned16(q_norm_weight) || !aligned16(k_norm_weight) || !aligned16(cos_sin) ||
       (k_out && !aligned16(k_out)) || (v_out && !aligned16(v_out)))
     return TLF_E_ALIGN;
   return TLF_OK;
@@ -447,8 +489,12 @@ extern "C" int tlf_qknorm_rope_store(const void *qkv, int64_t qkv_stride, const 
                           static_cast<unsigned short *>(v_out), static_cast<unsigned char *>(k_cache),
                           static_cast<unsigned char *>(v_cache), slot_mapping, num_slots, kv_dtype, k_scale,
                           v_scale, num_q_heads, num_kv_heads};
-  hipLaunchKernelGGL(qknorm_rope_store_kernel, dim3(n, (heads + 15) / 16), dim3(256), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const unsigned short *>(qkv), qkv_stride, a);
+  if (n >= 2048)   // a prefill step: 4 tokens per workgroup
+    hipLaunchKernelGGL(qknorm_rope_store_kernel<4>, dim3((n + 3) / 4, (heads + 15) / 16), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const unsigned short *>(qkv), qkv_stride, n, a);
+  else             // a decode step: as many workgroups as there are pieces of 16 heads
+    hipLaunchKernelGGL(qknorm_rope_store_kernel<1>, dim3(n, (heads + 15) / 16), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const unsigned short *>(qkv), qkv_stride, n, a);
   return launch_status();
 }
 
@@ -458,7 +504,7 @@ extern "C" int tlf_silu_and_mul(const void *x, void *y, int32_t rows, int32_t in
   if (rows < 0 || inter <= 0 || inter % 8) return TLF_E_SHAPE;
   if (!aligned16(x) || !aligned16(y)) return TLF_E_ALIGN;
   const int64_t total = static_cast<int64_t>(rows) * (inter / 8);
-  hipLaunchKernelGGL(silu_and_mul_kernel, dim3(static_cast<unsigned>((total + 255) / 256)),
+  hipLaunchKernelGGL(silu_and_mul_kernel, dim3(static_cast<unsigned>((total + 256 * kSiluUnroll - 1) / (256 * kSiluUnroll))),
                      dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<const unsigned short *>(x), static_cast<unsigned short *>(y),
                      static_cast<int64_t>(rows), inter);

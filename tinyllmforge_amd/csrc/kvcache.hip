@@ -1,8 +1,10 @@
 // Slot-mapped KV-cache write (reference: tinyvllm/layers/attention.py:9-48).
 //
-// One workgroup per token.  A K (or V) row is Hkv*Dh elements = 2 KiB in bf16:
-// the first half of the workgroup moves the K row, the second half the V row,
-// 16 bytes per lane, so every global access is a fully coalesced 128-bit one.
+// A K (or V) row is Hkv*Dh elements = 2 KiB in bf16: the first half of a workgroup moves K rows, the
+// second half V rows, 16 bytes per lane, so every global access is a fully coalesced 128-bit one.
+// A workgroup moves TOK consecutive tokens and a lane has all its TOK loads in flight before its first
+// store: with one token per workgroup the kernel is bound by load latency and by the rate at which
+// 4 KiB workgroups can be started, not by HBM.
 // HBM bound: 2 * row_bytes read + 2 * row_bytes written per token.
 #include "common.h"
 
@@ -10,21 +12,33 @@ namespace tlf {
 
 constexpr int kStoreThreads = 256;
 
+template <int TOK>
 __global__ __launch_bounds__(kStoreThreads) void store_kvcache_kernel(
     const unsigned char *__restrict__ key, int64_t key_stride,
     const unsigned char *__restrict__ value, int64_t value_stride,
     unsigned char *__restrict__ k_cache, unsigned char *__restrict__ v_cache,
-    const int32_t *__restrict__ slot_mapping, int32_t row_bytes, int64_t num_slots) {
-  const int token = blockIdx.x;
-  const int64_t slot = slot_mapping[token];
-  if (slot < 0 || slot >= num_slots) return;  // padding row: leave the cache alone
+    const int32_t *__restrict__ slot_mapping, int32_t num_tokens, int32_t row_bytes, int64_t num_slots) {
   const int half = kStoreThreads / 2;
   const bool is_v = threadIdx.x >= half;
   const int lane = is_v ? threadIdx.x - half : threadIdx.x;
-  const unsigned char *src = is_v ? value + token * value_stride : key + token * key_stride;
-  unsigned char *dst = (is_v ? v_cache : k_cache) + slot * static_cast<int64_t>(row_bytes);
+  const int64_t tok0 = static_cast<int64_t>(blockIdx.x) * TOK;
+  const unsigned char *src = is_v ? value : key;
+  const int64_t stride = is_v ? value_stride : key_stride;
+  unsigned char *cache = is_v ? v_cache : k_cache;
+  int64_t slot[TOK];
+#pragma unroll
+  for (int i = 0; i < TOK; ++i) {
+    slot[i] = tok0 + i < num_tokens ? slot_mapping[tok0 + i] : -1;
+    if (slot[i] >= num_slots) slot[i] = -1;   // padding row: leave the cache alone
+  }
   for (int off = lane * 16; off < row_bytes; off += half * 16) {
-    *reinterpret_cast<uint4 *>(dst + off) = *reinterpret_cast<const uint4 *>(src + off);
+    uint4 v[TOK];
+#pragma unroll
+    for (int i = 0; i < TOK; ++i)
+      if (slot[i] >= 0) v[i] = load_nt_u4(src + (tok0 + i) * stride + off);
+#pragma unroll
+    for (int i = 0; i < TOK; ++i)
+      if (slot[i] >= 0) *reinterpret_cast<uint4 *>(cache + slot[i] * static_cast<int64_t>(row_bytes) + off) = v[i];
   }
 }
 
@@ -75,11 +89,18 @@ extern "C" int tlf_store_kvcache(const void *key, int64_t key_stride_bytes, cons
       !aligned16(value) || !aligned16(k_cache) || !aligned16(v_cache))
     return TLF_E_ALIGN;
   if (key_stride_bytes < row_bytes || value_stride_bytes < row_bytes) return TLF_E_SHAPE;
-  hipLaunchKernelGGL(store_kvcache_kernel, dim3(num_tokens), dim3(kStoreThreads), 0,
-                     static_cast<hipStream_t>(stream), static_cast<const unsigned char *>(key),
-                     key_stride_bytes, static_cast<const unsigned char *>(value),
-                     value_stride_bytes, static_cast<unsigned char *>(k_cache),
-                     static_cast<unsigned char *>(v_cache), slot_mapping, row_bytes, num_slots);
+  if (num_tokens >= 2048)
+    hipLaunchKernelGGL(store_kvcache_kernel<8>, dim3((num_tokens + 7) / 8), dim3(kStoreThreads), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const unsigned char *>(key),
+                       key_stride_bytes, static_cast<const unsigned char *>(value),
+                       value_stride_bytes, static_cast<unsigned char *>(k_cache),
+                       static_cast<unsigned char *>(v_cache), slot_mapping, num_tokens, row_bytes, num_slots);
+  else
+    hipLaunchKernelGGL(store_kvcache_kernel<1>, dim3(num_tokens), dim3(kStoreThreads), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const unsigned char *>(key),
+                       key_stride_bytes, static_cast<const unsigned char *>(value),
+                       value_stride_bytes, static_cast<unsigned char *>(k_cache),
+                       static_cast<unsigned char *>(v_cache), slot_mapping, num_tokens, row_bytes, num_slots);
   return launch_status();
 }
 

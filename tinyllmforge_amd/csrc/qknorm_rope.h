@@ -30,20 +30,57 @@ struct QkRopeStoreArgs {
 
 // (reference op sequence: tinyvllm/models/qwen3.py:79-94, layers/attention.py:94-95)
 // 16 lanes own one head (8 dims each); lanes j < 8 hold the first half of the head, lanes j >= 8 the second,
-// so the RoPE partner of lane j is lane j ^ 8.  raw = this lane's 8 bf16 values of token tok, head `head`
-// (q heads first, then k, then v); all 16 lanes of a head call together.
-__device__ __forceinline__ void qknorm_rope_store_piece(const uint4 raw, int64_t tok, int head, int j,
-                                                        const QkRopeStoreArgs &a) {
+// so the RoPE partner of lane j is lane j ^ 8.  The work on one 8-value piece comes in three steps, so that a
+// kernel that handles several tokens per lane can issue every step's loads for all of them before it waits:
+//   1. qk_piece_meta: the token's position and cache slot (one load each);
+//   2. qk_piece_table: this lane's 8 cosines and 8 sines of that position (q and k heads only);
+//   3. qk_piece_finish: norm, rotation and the stores.
+struct QkPieceMeta {
+  int64_t pos;    // the token's position (q and k heads)
+  int64_t slot;   // cache slot of the token, or -1: no cache store (k and v heads)
+};
+struct QkPieceTable {
+  float4 c0, c1, s0, s1;   // cos[8], sin[8] of this lane's dims
+};
+
+__device__ __forceinline__ QkPieceMeta qk_piece_meta(int64_t tok, int head, const QkRopeStoreArgs &a) {
+  QkPieceMeta m;
+  m.pos = 0;
+  m.slot = -1;
+  const bool is_q = head < a.num_q_heads;
+  const bool is_v = head >= a.num_q_heads + a.num_kv_heads;
+  if (!is_v) m.pos = a.positions[tok];
+  if (!is_q && a.slot_mapping != nullptr) {
+    m.slot = a.slot_mapping[tok];
+    if (m.slot >= a.num_slots) m.slot = -1;
+  }
+  return m;
+}
+
+__device__ __forceinline__ QkPieceTable qk_piece_table(const QkPieceMeta &m, int head, int j, const QkRopeStoreArgs &a) {
+  QkPieceTable t;
+  t.c0 = t.c1 = t.s0 = t.s1 = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (head < a.num_q_heads + a.num_kv_heads) {
+    const bool pos_ok = m.pos >= 0 && m.pos < a.max_pos;
+    const float *cs = a.cos_sin + (pos_ok ? m.pos : 0) * 128 + (j % 8) * 8;
+    t.c0 = *reinterpret_cast<const float4 *>(cs);
+    t.c1 = *reinterpret_cast<const float4 *>(cs + 4);
+    t.s0 = *reinterpret_cast<const float4 *>(cs + 64);
+    t.s1 = *reinterpret_cast<const float4 *>(cs + 68);
+  }
+  return t;
+}
+
+// raw = this lane's 8 bf16 values of token tok, head `head` (q heads first, then k, then v); all 16 lanes of
+// a head call together.
+__device__ __forceinline__ void qk_piece_finish(const uint4 raw, int64_t tok, int head, int j, const QkPieceMeta &m,
+                                                const QkPieceTable &t, const QkRopeStoreArgs &a) {
   constexpr int kDh = 128;
   const int num_q_heads = a.num_q_heads, num_kv_heads = a.num_kv_heads;
   const bool is_q = head < num_q_heads;
   const bool is_k = !is_q && head < num_q_heads + num_kv_heads;
   const int kvh = is_q ? 0 : (is_k ? head - num_q_heads : head - num_q_heads - num_kv_heads);
-  int64_t slot = -1;
-  if (!is_q && a.slot_mapping != nullptr) {
-    slot = a.slot_mapping[tok];
-    if (slot >= a.num_slots) slot = -1;
-  }
+  const int64_t slot = m.slot;
   uint4 outp = raw;
   if (is_q || is_k) {
     float v[8];
@@ -51,8 +88,13 @@ __device__ __forceinline__ void qknorm_rope_store_piece(const uint4 raw, int64_t
     float ss = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) ss = fmaf(v[i], v[i], ss);
-#pragma unroll
-    for (int o = 8; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    // sum over the head's 16 lanes: rotations by 8, 4, 2, 1 inside the row add the same pairs, in the same
+    // order, as a butterfly over lane ^ 8, 4, 2, 1 would (after each step the partial sums repeat with that
+    // period), so every lane of the head ends with the same bits
+    ss += row_ror<8>(ss);
+    ss += row_ror<4>(ss);
+    ss += row_ror<2>(ss);
+    ss += row_ror<1>(ss);
     const float inv = 1.0f / sqrtf(ss / static_cast<float>(kDh) + a.eps);
     float w[8];
     unpack8(*reinterpret_cast<const uint4 *>((is_q ? a.qw : a.kw) + j * 8), w);
@@ -63,19 +105,16 @@ __device__ __forceinline__ void qknorm_rope_store_piece(const uint4 raw, int64_t
       nrm[i] = bf16_bits_to_float(float_to_bf16_bits(__fmul_rn(nn, w[i])));
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) other[i] = __shfl_xor(nrm[i], 8, 64);
-    const int64_t pos = a.positions[tok];
-    const bool pos_ok = pos >= 0 && pos < a.max_pos;
-    const float *cs = a.cos_sin + (pos_ok ? pos : 0) * kDh;
-    const int cj = (j % 8) * 8;
+    for (int i = 0; i < 8; ++i) other[i] = row_ror<8>(nrm[i]);   // lane j ^ 8
+    const bool pos_ok = m.pos >= 0 && m.pos < a.max_pos;
+    const float cosv[8] = {t.c0.x, t.c0.y, t.c0.z, t.c0.w, t.c1.x, t.c1.y, t.c1.z, t.c1.w};
+    const float sinv[8] = {t.s0.x, t.s0.y, t.s0.z, t.s0.w, t.s1.x, t.s1.y, t.s1.z, t.s1.w};
     float o[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const float co = cs[cj + i];
-      const float si = cs[64 + cj + i];
       // lanes j < 8: cos*x1 - sin*x2 ; lanes j >= 8: cos*x2 + sin*x1
-      const float x = __fmul_rn(co, nrm[i]);
-      const float y = __fmul_rn(si, other[i]);
+      const float x = __fmul_rn(cosv[i], nrm[i]);
+      const float y = __fmul_rn(sinv[i], other[i]);
       o[i] = (j < 8) ? __fsub_rn(x, y) : __fadd_rn(x, y);
       if (!pos_ok) o[i] = nrm[i];
     }
@@ -105,6 +144,14 @@ __device__ __forceinline__ void qknorm_rope_store_piece(const uint4 raw, int64_t
     hi = __builtin_amdgcn_cvt_pk_fp8_f32(f[6], f[7], hi, true);
     *reinterpret_cast<int2 *>(cache + slot * row_elems + kvh * kDh + j * 8) = make_int2(lo, hi);
   }
+}
+
+// The three steps on one piece.
+__device__ __forceinline__ void qknorm_rope_store_piece(const uint4 raw, int64_t tok, int head, int j,
+                                                        const QkRopeStoreArgs &a) {
+  const QkPieceMeta m = qk_piece_meta(tok, head, a);
+  const QkPieceTable t = qk_piece_table(m, head, j, a);
+  qk_piece_finish(raw, tok, head, j, m, t, a);
 }
 
 // Argument checks shared by the entry points that end in this step; fills `a` (q_out .. v_scale as given).
