@@ -570,6 +570,19 @@ def bench_e2e(args, quantization):
         slice_steps, slice_s = args.steps, at_mark
     else:
         slice_steps, slice_s = all_steps, wall
+    mr = llm.model_runner
+    if getattr(mr, "graph_kernels", None):
+        # kernels of one decode step: the captured graph of the largest batch bucket plus the LM head + argmax
+        # that follow it (counted by the library around one call)
+        from tinyllmforge_amd import _lib
+        lib = _lib.load()
+        top = max(mr.graph_kernels)
+        before = lib.tlf_kernel_launches()
+        mr.model.compute_greedy_ids(mr.graph_vars["outputs"][:top])
+        torch.cuda.synchronize()
+        stats["kernels_per_decode_step"] = dict(batch_bucket=top, in_graph=mr.graph_kernels[top],
+                                                lm_head_and_argmax=lib.tlf_kernel_launches() - before,
+                                                layers=llm.config.hf_config.num_hidden_layers)
     res = dict(tok_s=total / wall, wall_s=wall, total_output_tokens=total, init_s=round(init_s, 1), stats=stats,
                kv_blocks=llm.config.num_kvcache_blocks, slice_steps=slice_steps, slice_s=slice_s)
     if quantization is not None:

@@ -51,6 +51,10 @@ const char *tlf_error_string(int code);
 /* Multiprocessor count and LDS bytes per workgroup of the current device
  * (host query; either out pointer may be NULL). */
 int tlf_device_info(int32_t *num_cus, int32_t *lds_bytes);
+/* Number of kernels this library has launched in this process so far (host counter, every entry point).
+ * A statistic for benchmarks: read it before and after one eager engine step, or around a graph capture,
+ * to count the kernels of a step.  No counterpart in the reference. */
+int64_t tlf_kernel_launches(void);
 
 /* ---------------------------------------------------------------------------
  * a1  store_kvcache   replaces layers/attention.py:33-48 (Triton kernel 9-30)

@@ -24,6 +24,7 @@ SIGNATURES = {
     "tlf_version": (c_int32, []),
     "tlf_error_string": (c_char_p, [c_int32]),
     "tlf_device_info": (c_int32, [_P, _P]),
+    "tlf_kernel_launches": (c_int64, []),
     "tlf_store_kvcache": (c_int32, [_P, _I64, _P, _I64, _P, _P, _P, _I32, _I32, _I64, _P]),
     "tlf_store_kvcache_fp8": (c_int32, [_P, _I64, _P, _I64, _P, _P, _P, _I32, _I32, _I32, _P, _P, _I64, _P]),
     "tlf_rmsnorm": (c_int32, [_P, _I64, _P, _P, _I32, _I32, _I32, _F, _P]),

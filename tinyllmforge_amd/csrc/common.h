@@ -1,5 +1,6 @@
 // Shared device/host helpers for the gfx950 kernels of libtlf_hip.so.
 #pragma once
+#include <atomic>
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -231,6 +232,15 @@ int launch_argmax_final(const unsigned long long *keys, int32_t nparts, int64_t 
                         hipStream_t stream);
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Kernels this library has launched in this process: a statistic for benchmarks (kernels per engine step are
+// counted around one eager step or one graph capture); every launch of the library goes through TLF_LAUNCH.
+extern std::atomic<long long> g_kernel_launches;
+#define TLF_LAUNCH(...)                                                      \
+  do {                                                                       \
+    tlf::g_kernel_launches.fetch_add(1, std::memory_order_relaxed);          \
+    hipLaunchKernelGGL(__VA_ARGS__);                                         \
+  } while (0)
 
 inline int launch_status() {
   hipError_t e = hipGetLastError();

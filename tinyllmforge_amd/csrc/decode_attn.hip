@@ -654,9 +654,9 @@ extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void
   // e4m3 rows: two tiles per trip where the bf16 image of both fits LDS (up to 8 KV heads)
 #define TLF_DECODE(NW)                                                                              \
   if (f8)                                                                                           \
-    hipLaunchKernelGGL((paged_decode_kernel<NW, true, (NW <= 8 ? 2 : 1)>), g, dim3(NW * 64), 0, s, p); \
+    TLF_LAUNCH((paged_decode_kernel<NW, true, (NW <= 8 ? 2 : 1)>), g, dim3(NW * 64), 0, s, p); \
   else                                                                                              \
-    hipLaunchKernelGGL((paged_decode_kernel<NW, false, 1>), g, dim3(NW * 64), 0, s, p)
+    TLF_LAUNCH((paged_decode_kernel<NW, false, 1>), g, dim3(NW * 64), 0, s, p)
   switch (num_kv_heads) {
     case 1: TLF_DECODE(1); break;
     case 2: TLF_DECODE(2); break;
@@ -668,6 +668,6 @@ extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void
 #undef TLF_DECODE
   int rc = launch_status();
   if (rc != TLF_OK) return rc;
-  hipLaunchKernelGGL(paged_decode_merge_kernel, dim3((num_q_heads + 7) / 8, batch), dim3(256), 0, s, p);
+  TLF_LAUNCH(paged_decode_merge_kernel, dim3((num_q_heads + 7) / 8, batch), dim3(256), 0, s, p);
   return launch_status();
 }

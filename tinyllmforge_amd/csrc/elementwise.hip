@@ -65,7 +65,7 @@ int launch_rmsnorm(const void *x, int64_t x_outer_stride, const void *residual, 
   auto ys = static_cast<unsigned short *>(y);
   auto ro = static_cast<unsigned short *>(residual_out);
 #define TLF_RMS(TPR, MAXC)                                                                       \
-  hipLaunchKernelGGL((rmsnorm_kernel<TPR, MAXC, ADD>),                                            \
+  TLF_LAUNCH((rmsnorm_kernel<TPR, MAXC, ADD>),                                            \
                      dim3(static_cast<unsigned>((rows + (256 / TPR) - 1) / (256 / TPR))),         \
                      dim3(256), 0, stream, xs, x_outer_stride, rs, ws, ys, ro, rows, inner, cols, \
                      eps)
@@ -370,9 +370,9 @@ __global__ __launch_bounds__(256) void sample_partial_kernel(
 int launch_argmax_final(const unsigned long long *keys, int32_t nparts, int64_t *out, int32_t rows,
                         hipStream_t stream) {
   if (nparts > 256)  // the keys of an LM-head epilogue: thousands per row
-    hipLaunchKernelGGL(argmax_final_kernel<256>, dim3(rows), dim3(256), 0, stream, keys, nparts, out);
+    TLF_LAUNCH(argmax_final_kernel<256>, dim3(rows), dim3(256), 0, stream, keys, nparts, out);
   else
-    hipLaunchKernelGGL(argmax_final_kernel<64>, dim3(rows), dim3(64), 0, stream, keys, nparts, out);
+    TLF_LAUNCH(argmax_final_kernel<64>, dim3(rows), dim3(64), 0, stream, keys, nparts, out);
   return launch_status();
 }
 
@@ -431,7 +431,7 @@ extern "C" int tlf_rope(const int64_t *positions, const void *q, int64_t q_strid
       k_stride % 8)
     return TLF_E_ALIGN;
   const int64_t total = static_cast<int64_t>(n) * (num_q_heads + num_kv_heads) * (head_dim / 16);
-  hipLaunchKernelGGL(rope_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
+  TLF_LAUNCH(rope_kernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), positions,
                      static_cast<const unsigned short *>(q), q_stride,
                      static_cast<const unsigned short *>(k), k_stride, cos_sin,
@@ -490,10 +490,10 @@ extern "C" int tlf_qknorm_rope_store(const void *qkv, int64_t qkv_stride, const 
                           static_cast<unsigned char *>(v_cache), slot_mapping, num_slots, kv_dtype, k_scale,
                           v_scale, num_q_heads, num_kv_heads};
   if (n >= 2048)   // a prefill step: 4 tokens per workgroup
-    hipLaunchKernelGGL(qknorm_rope_store_kernel<4>, dim3((n + 3) / 4, (heads + 15) / 16), dim3(256), 0,
+    TLF_LAUNCH(qknorm_rope_store_kernel<4>, dim3((n + 3) / 4, (heads + 15) / 16), dim3(256), 0,
                        static_cast<hipStream_t>(stream), static_cast<const unsigned short *>(qkv), qkv_stride, n, a);
   else             // a decode step: as many workgroups as there are pieces of 16 heads
-    hipLaunchKernelGGL(qknorm_rope_store_kernel<1>, dim3(n, (heads + 15) / 16), dim3(256), 0,
+    TLF_LAUNCH(qknorm_rope_store_kernel<1>, dim3(n, (heads + 15) / 16), dim3(256), 0,
                        static_cast<hipStream_t>(stream), static_cast<const unsigned short *>(qkv), qkv_stride, n, a);
   return launch_status();
 }
@@ -504,7 +504,7 @@ extern "C" int tlf_silu_and_mul(const void *x, void *y, int32_t rows, int32_t in
   if (rows < 0 || inter <= 0 || inter % 8) return TLF_E_SHAPE;
   if (!aligned16(x) || !aligned16(y)) return TLF_E_ALIGN;
   const int64_t total = static_cast<int64_t>(rows) * (inter / 8);
-  hipLaunchKernelGGL(silu_and_mul_kernel, dim3(static_cast<unsigned>((total + 256 * kSiluUnroll - 1) / (256 * kSiluUnroll))),
+  TLF_LAUNCH(silu_and_mul_kernel, dim3(static_cast<unsigned>((total + 256 * kSiluUnroll - 1) / (256 * kSiluUnroll))),
                      dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<const unsigned short *>(x), static_cast<unsigned short *>(y),
                      static_cast<int64_t>(rows), inter);
@@ -517,7 +517,7 @@ extern "C" int tlf_embedding(const int64_t *ids, const void *weight, void *y, in
   if (!ids || !weight || !y) return TLF_E_NULL;
   if (n < 0 || vocab <= 0 || cols <= 0 || cols % 8) return TLF_E_SHAPE;
   if (!aligned16(weight) || !aligned16(y)) return TLF_E_ALIGN;
-  hipLaunchKernelGGL(embedding_kernel, dim3(n), dim3(256), 0, static_cast<hipStream_t>(stream), ids,
+  TLF_LAUNCH(embedding_kernel, dim3(n), dim3(256), 0, static_cast<hipStream_t>(stream), ids,
                      static_cast<const unsigned short *>(weight), static_cast<unsigned short *>(y),
                      vocab, cols);
   return launch_status();
@@ -540,10 +540,10 @@ extern "C" int tlf_argmax(const void *logits, int64_t row_stride, int64_t *out, 
     return TLF_E_WORKSPACE;
   const int nchunks = argmax_chunks(rows, vocab);
   auto part = static_cast<unsigned long long *>(workspace);
-  hipLaunchKernelGGL(argmax_partial_kernel, dim3(nchunks, rows), dim3(256), 0,
+  TLF_LAUNCH(argmax_partial_kernel, dim3(nchunks, rows), dim3(256), 0,
                      static_cast<hipStream_t>(stream),
                      static_cast<const unsigned short *>(logits), row_stride, vocab, part, nchunks);
-  hipLaunchKernelGGL(argmax_final_kernel<64>, dim3(rows), dim3(64), 0,
+  TLF_LAUNCH(argmax_final_kernel<64>, dim3(rows), dim3(64), 0,
                      static_cast<hipStream_t>(stream), part, nchunks, out);
   return launch_status();
 }
@@ -593,10 +593,10 @@ extern "C" int tlf_argmax_noalloc(const void *logits, int64_t row_stride, int64_
   // every (row, chunk) key that the second kernel reads is written by the first one in this call:
   // nothing of an earlier call's contents is read, so the array needs no clearing
   const int nchunks = argmax_chunks(rows, vocab);
-  hipLaunchKernelGGL(argmax_partial_kernel, dim3(nchunks, rows), dim3(256), 0,
+  TLF_LAUNCH(argmax_partial_kernel, dim3(nchunks, rows), dim3(256), 0,
                      static_cast<hipStream_t>(stream),
                      static_cast<const unsigned short *>(logits), row_stride, vocab, part, nchunks);
-  hipLaunchKernelGGL(argmax_final_kernel<64>, dim3(rows), dim3(64), 0,
+  TLF_LAUNCH(argmax_final_kernel<64>, dim3(rows), dim3(64), 0,
                      static_cast<hipStream_t>(stream), part, nchunks, out);
   return launch_status();
 }
@@ -613,12 +613,12 @@ extern "C" int tlf_sample(const void *logits, int64_t row_stride, const float *t
     return TLF_E_WORKSPACE;
   const int nchunks = argmax_chunks(rows, vocab);
   auto part = static_cast<unsigned long long *>(workspace);
-  hipLaunchKernelGGL(sample_partial_kernel, dim3(nchunks, rows), dim3(256), 0,
+  TLF_LAUNCH(sample_partial_kernel, dim3(nchunks, rows), dim3(256), 0,
                      static_cast<hipStream_t>(stream), static_cast<const unsigned short *>(logits),
                      row_stride, vocab, temperatures, static_cast<unsigned int>(seed),
                      static_cast<unsigned int>(seed >> 32), static_cast<unsigned int>(offset),
                      static_cast<unsigned int>(offset >> 32), part, nchunks);
-  hipLaunchKernelGGL(argmax_final_kernel<64>, dim3(rows), dim3(64), 0,
+  TLF_LAUNCH(argmax_final_kernel<64>, dim3(rows), dim3(64), 0,
                      static_cast<hipStream_t>(stream), part, nchunks, out);
   return launch_status();
 }

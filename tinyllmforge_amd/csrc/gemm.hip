@@ -1020,9 +1020,9 @@ int launch_skinny(const GemmParams &p, hipStream_t stream) {
   const int pipe_m = gemm_tuning().skinny_pipe_m >= 0 ? gemm_tuning().skinny_pipe_m : tiles16 <= 256 ? 8 : 4;
 #define TLF_SK(MT_, TN_)                                                                                 \
   if (MT_ == 1 && p.M <= pipe_m)                                                                         \
-    hipLaunchKernelGGL((skinny_gemm_kernel<MT_, TN_, W8, MT_ == 1>), grid, dim3(512), 0, stream, p);     \
+    TLF_LAUNCH((skinny_gemm_kernel<MT_, TN_, W8, MT_ == 1>), grid, dim3(512), 0, stream, p);     \
   else                                                                                                   \
-    hipLaunchKernelGGL((skinny_gemm_kernel<MT_, TN_, W8, false>), grid, dim3(512), 0, stream, p)
+    TLF_LAUNCH((skinny_gemm_kernel<MT_, TN_, W8, false>), grid, dim3(512), 0, stream, p)
 #define TLF_SK_TN(MT_)      \
   if (tn == 4) {            \
     TLF_SK(MT_, 4);         \
@@ -1327,7 +1327,7 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
 #define TLF_WS(TM_, NS_, PF_, KG_, COLS_)                                                           \
   if (!launched && g.bm == TM_ * 32 && g.kgroups == KG_ && g.bn == COLS_ * 32) {                    \
     if (!dry)                                                                                       \
-      hipLaunchKernelGGL((gemm_wstream_kernel<TM_, NS_, PF_, KG_, COLS_>), wgrid,                   \
+      TLF_LAUNCH((gemm_wstream_kernel<TM_, NS_, PF_, KG_, COLS_>), wgrid,                   \
                          dim3((COLS_ * KG_ + 1) * 64), 0, stream, p);                               \
     launched = true;                                                                                \
   }
@@ -1346,7 +1346,7 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
       g.kgroups == KG_ && (g.wn == 0 || g.wn == WN_)) {                                                                   \
     p.amax_parts = p.n_tiles * WN_;                                                         \
     if (!dry)                                                                               \
-      hipLaunchKernelGGL((gemm_dlds_kernel<BN_, BM_, WN_, WM_, W8, NS_, OCC_, KG_>), grid,  \
+      TLF_LAUNCH((gemm_dlds_kernel<BN_, BM_, WN_, WM_, W8, NS_, OCC_, KG_>), grid,  \
                          dim3(WN_ * WM_ * KG_ * 64), 0, stream, p);                         \
     launched = true;                                                                        \
   }
@@ -1388,7 +1388,7 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   if (g.splits > 1) {
     if (tail) {  // the caller checked that this plan splits K and that the row fits the kernel
 #define TLF_TAIL(TPR_, MAXC_)                                                                 \
-  hipLaunchKernelGGL((splitk_reduce_add_rmsnorm_kernel<TPR_, MAXC_, W8>),                     \
+  TLF_LAUNCH((splitk_reduce_add_rmsnorm_kernel<TPR_, MAXC_, W8>),                     \
                      dim3(static_cast<unsigned>((M + (256 / TPR_) - 1) / (256 / TPR_))), dim3(256), 0, \
                      stream, p, *tail)
       TLF_RMS_SHAPES(N, TLF_TAIL);
@@ -1396,13 +1396,13 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
       return launch_status();
     }
     if (qk) {  // likewise: N = (Hq + 2 Hkv) * 128
-      hipLaunchKernelGGL((splitk_reduce_qknorm_rope_store_kernel<W8>),
+      TLF_LAUNCH((splitk_reduce_qknorm_rope_store_kernel<W8>),
                          dim3(static_cast<unsigned>(M), static_cast<unsigned>((N / 128 + 15) / 16)), dim3(256), 0,
                          stream, p, *qk);
       return launch_status();
     }
     const int64_t total4 = static_cast<int64_t>(M) * N / 4;
-    hipLaunchKernelGGL((splitk_reduce_kernel<W8>), dim3(static_cast<unsigned>((total4 + 255) / 256)),
+    TLF_LAUNCH((splitk_reduce_kernel<W8>), dim3(static_cast<unsigned>((total4 + 255) / 256)),
                        dim3(256), 0, stream, p);
     rc = launch_status();
   }
@@ -1501,7 +1501,7 @@ extern "C" int tlf_w8a16_pack_weight(const void *wq_rowmajor, void *packed, int3
   if (!aligned16(wq_rowmajor) || !aligned16(packed)) return TLF_E_ALIGN;
   if (wq_rowmajor == packed) return TLF_E_UNSUPPORTED;  // not in place
   const int64_t atoms = static_cast<int64_t>(tlf_w8a16_packed_bytes(N, K) / 16);
-  hipLaunchKernelGGL(pack_w8_kernel, dim3(static_cast<unsigned>((atoms + 255) / 256)), dim3(256), 0,
+  TLF_LAUNCH(pack_w8_kernel, dim3(static_cast<unsigned>((atoms + 255) / 256)), dim3(256), 0,
                      static_cast<hipStream_t>(stream), static_cast<const uint4 *>(wq_rowmajor),
                      static_cast<uint4 *>(packed), N, K, atoms);
   return launch_status();

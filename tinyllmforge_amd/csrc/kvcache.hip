@@ -90,13 +90,13 @@ extern "C" int tlf_store_kvcache(const void *key, int64_t key_stride_bytes, cons
     return TLF_E_ALIGN;
   if (key_stride_bytes < row_bytes || value_stride_bytes < row_bytes) return TLF_E_SHAPE;
   if (num_tokens >= 2048)
-    hipLaunchKernelGGL(store_kvcache_kernel<8>, dim3((num_tokens + 7) / 8), dim3(kStoreThreads), 0,
+    TLF_LAUNCH(store_kvcache_kernel<8>, dim3((num_tokens + 7) / 8), dim3(kStoreThreads), 0,
                        static_cast<hipStream_t>(stream), static_cast<const unsigned char *>(key),
                        key_stride_bytes, static_cast<const unsigned char *>(value),
                        value_stride_bytes, static_cast<unsigned char *>(k_cache),
                        static_cast<unsigned char *>(v_cache), slot_mapping, num_tokens, row_bytes, num_slots);
   else
-    hipLaunchKernelGGL(store_kvcache_kernel<1>, dim3(num_tokens), dim3(kStoreThreads), 0,
+    TLF_LAUNCH(store_kvcache_kernel<1>, dim3(num_tokens), dim3(kStoreThreads), 0,
                        static_cast<hipStream_t>(stream), static_cast<const unsigned char *>(key),
                        key_stride_bytes, static_cast<const unsigned char *>(value),
                        value_stride_bytes, static_cast<unsigned char *>(k_cache),
@@ -120,7 +120,7 @@ extern "C" int tlf_store_kvcache_fp8(const void *key, int64_t key_stride_bytes, 
       (reinterpret_cast<uintptr_t>(k_cache) & 7u) || (reinterpret_cast<uintptr_t>(v_cache) & 7u))
     return TLF_E_ALIGN;
   if (key_stride_bytes < row_bytes_in || value_stride_bytes < row_bytes_in) return TLF_E_SHAPE;
-  hipLaunchKernelGGL(store_kvcache_fp8_kernel, dim3(num_tokens), dim3(kStoreThreads), 0,
+  TLF_LAUNCH(store_kvcache_fp8_kernel, dim3(num_tokens), dim3(kStoreThreads), 0,
                      static_cast<hipStream_t>(stream), static_cast<const unsigned char *>(key),
                      key_stride_bytes, static_cast<const unsigned char *>(value),
                      value_stride_bytes, static_cast<unsigned char *>(k_cache),

@@ -1,7 +1,13 @@
 // Library-level entry points of libtlf_hip.so.
 #include "common.h"
 
+namespace tlf {
+std::atomic<long long> g_kernel_launches{0};
+}
+
 extern "C" int tlf_version(void) { return TLF_ABI_VERSION; }
+
+extern "C" int64_t tlf_kernel_launches(void) { return tlf::g_kernel_launches.load(std::memory_order_relaxed); }
 
 extern "C" const char *tlf_error_string(int code) {
   switch (code) {
@@ -142,7 +148,7 @@ extern "C" int tlf_probe_mfma(void *out, int32_t iters, int32_t mode, void *stre
   if (!out) return TLF_E_NULL;
   if (iters < 0 || (mode != 0 && mode != 1)) return TLF_E_SHAPE;
   // one workgroup of four waves per CU slot, twice the CUs: two waves per SIMD keep the pipe full
-  hipLaunchKernelGGL(tlf::probe_mfma_kernel, dim3(512), dim3(256), 0, static_cast<hipStream_t>(stream),
+  TLF_LAUNCH(tlf::probe_mfma_kernel, dim3(512), dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<float *>(out), iters, mode);
   return tlf::launch_status();
 }
@@ -153,7 +159,7 @@ extern "C" int tlf_probe_mix(const void *big, size_t big_bytes, const void *smal
   if (!tlf::aligned16(big) || !tlf::aligned16(small_region)) return TLF_E_ALIGN;
   const size_t kib_per_wave = big_bytes / 1024 / (256 * 4) / 16 * 16;
   if (kib_per_wave == 0 || small_bytes < 16 * 1024 || small_bytes % 1024 || l2_eighths < 0) return TLF_E_SHAPE;
-  hipLaunchKernelGGL(tlf::probe_mix_kernel, dim3(256), dim3(512), 0, static_cast<hipStream_t>(stream),
+  TLF_LAUNCH(tlf::probe_mix_kernel, dim3(256), dim3(512), 0, static_cast<hipStream_t>(stream),
                      static_cast<const unsigned char *>(big), kib_per_wave,
                      static_cast<const unsigned char *>(small_region), small_bytes / 1024, l2_eighths,
                      static_cast<unsigned int *>(sink));
@@ -164,7 +170,7 @@ extern "C" int tlf_probe_read(const void *src, size_t bytes, void *sink, void *s
   if (!src || !sink) return TLF_E_NULL;
   if (bytes % 16 || !tlf::aligned16(src)) return TLF_E_ALIGN;
   if (bytes == 0) return TLF_OK;
-  hipLaunchKernelGGL(tlf::probe_read_kernel, dim3(256), dim3(256), 0,
+  TLF_LAUNCH(tlf::probe_read_kernel, dim3(256), dim3(256), 0,
                      static_cast<hipStream_t>(stream), static_cast<const uint4 *>(src), bytes / 16,
                      static_cast<unsigned int *>(sink));
   return tlf::launch_status();
@@ -174,7 +180,7 @@ extern "C" int tlf_probe_copy(const void *src, void *dst, size_t bytes, void *st
   if (!src || !dst) return TLF_E_NULL;
   if (bytes % 16 || !tlf::aligned16(src) || !tlf::aligned16(dst)) return TLF_E_ALIGN;
   if (bytes == 0) return TLF_OK;
-  hipLaunchKernelGGL(tlf::probe_copy_kernel, dim3(256 * 8), dim3(256), 0,
+  TLF_LAUNCH(tlf::probe_copy_kernel, dim3(256 * 8), dim3(256), 0,
                      static_cast<hipStream_t>(stream), static_cast<const uint4 *>(src),
                      static_cast<uint4 *>(dst), bytes / 16);
   return tlf::launch_status();

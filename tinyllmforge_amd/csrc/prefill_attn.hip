@@ -574,11 +574,11 @@ extern "C" int tlf_varlen_prefill_attn(const void *q, int64_t q_stride, const vo
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (paged && kv_dtype == TLF_KV_FP8_E4M3) {
     // the K scale is a per-head constant of the scores: fold it in on the device side per head
-    if (nwv == 8) hipLaunchKernelGGL((prefill_attn_kernel<CT, true, 8>), grid, dim3(512), 0, s, p);
-    else hipLaunchKernelGGL((prefill_attn_kernel<CT, true, 4>), grid, dim3(256), 0, s, p);
+    if (nwv == 8) TLF_LAUNCH((prefill_attn_kernel<CT, true, 8>), grid, dim3(512), 0, s, p);
+    else TLF_LAUNCH((prefill_attn_kernel<CT, true, 4>), grid, dim3(256), 0, s, p);
   } else {
-    if (nwv == 8) hipLaunchKernelGGL((prefill_attn_kernel<CT, false, 8>), grid, dim3(512), 0, s, p);
-    else hipLaunchKernelGGL((prefill_attn_kernel<CT, false, 4>), grid, dim3(256), 0, s, p);
+    if (nwv == 8) TLF_LAUNCH((prefill_attn_kernel<CT, false, 8>), grid, dim3(512), 0, s, p);
+    else TLF_LAUNCH((prefill_attn_kernel<CT, false, 4>), grid, dim3(256), 0, s, p);
   }
   return launch_status();
 }

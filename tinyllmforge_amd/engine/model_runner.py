@@ -11,6 +11,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
+from .. import _lib
 from ..config import Config
 from ..layers.sampler import Sampler
 from ..models.qwen3 import Qwen3ForCausalLM
@@ -316,13 +317,17 @@ class ModelRunner:
         self.graph_max_blocks = max_blocks
         self.graph_bs = [b for b in (1, 2, 4, 8) if b <= max_bs] + list(range(16, max_bs + 1, 16))
         pool = None
+        lib = _lib.load()
+        self.graph_kernels = {}      # batch bucket -> kernels in its graph
         for bs in reversed(self.graph_bs):
             graph = torch.cuda.CUDAGraph()
             set_context(False, slot_mapping=gv["slot_mapping"][:bs], context_lens=gv["context_lens"][:bs],
                         block_tables=gv["block_tables"][:bs, :])
             gv["outputs"][:bs] = self.model(gv["input_ids"][:bs], gv["positions"][:bs])    # warm-up
+            launched = lib.tlf_kernel_launches()
             with torch.cuda.graph(graph, pool):
                 gv["outputs"][:bs] = self.model(gv["input_ids"][:bs], gv["positions"][:bs])
+            self.graph_kernels[bs] = lib.tlf_kernel_launches() - launched + 1    # + the copy into the static output
             if pool is None:
                 pool = graph.pool()
             self.graphs[bs] = graph
