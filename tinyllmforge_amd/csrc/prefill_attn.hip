@@ -27,10 +27,13 @@
 //    weight below 2^-14 would be an fp16 subnormal, and a row with one dominant key and thousands of faint ones
 //    would lose their mass from the numerator but not from the denominator.
 //  - a bf16 V tile that fp16 cannot hold (some |v| >= 65536, or no element as large as 2^-9, where the whole
-//    tile would sit in or near the subnormal range) is staged as it is and multiplied in bf16, with P as a
-//    bf16 hi + lo pair: the choice is made per 64-token tile from a vote of the staging threads.  A tile with
-//    some |v| >= 2^112, where 2^15 p v could leave fp32, ends the 2^15 carry for the rest of the row tile
-//    (accumulators and sums are scaled back once, every later tile is multiplied in bf16).
+//    tile would sit in or near the subnormal range) ends the workgroup: the staging threads vote on every
+//    64-token tile, and on such a tile the workgroup writes a marker (a NaN pattern no arithmetic produces) into
+//    the first output element of its row tile and leaves.  A second launch of the same grid (MODE 1) looks at
+//    that element, returns at once where the marker is absent, and otherwise computes the row tile again with
+//    both products in bf16 (P as a bf16 hi + lo pair, no 2^15 factor), which holds whatever bf16 holds.  Real
+//    checkpoints never take it; keeping it in a launch of its own keeps its registers and branches out of the
+//    fp16 kernel (inside one kernel the same choice cost 20-30 % on every call).
 #include <stdlib.h>
 
 #include "common.h"
@@ -82,7 +85,7 @@ constexpr float kPShift = 15.0f;          // P is carried as 2^15 p
 // bf16 bit patterns (sign cleared) that bound what a tile may hold for the fp16 product
 constexpr unsigned int kVBigBits = 0x4780u;     // 65536: the first bf16 above the largest finite fp16
 constexpr unsigned int kVDecentBits = 0x3b00u;  // 2^-9
-constexpr unsigned int kVHugeBits = 0x7780u;    // 2^112: 2^15 p v may overflow fp32 from here on
+constexpr unsigned short kRedoMarker = 0xffa5u;  // bf16 NaN with a payload: "compute this row tile again in bf16"
 typedef unsigned short ushortx2 __attribute__((ext_vector_type(2)));
 
 struct PrefillParams {
@@ -154,9 +157,13 @@ __device__ __forceinline__ void rescale16(floatx4 (&acc)[8], int d0, float alpha
   for (int e = 0; e < 16; ++e) acc[d0 + e / 4][e % 4] = t[e];
 }
 
-template <int CT, bool KV8, int NWV>
+// MODE 0: second product in fp16 (bf16 rows: leaves a marker and returns on a tile fp16 cannot hold);
+// MODE 1 (bf16 rows only): both products in bf16, for the row tiles that carry the marker.
+template <int CT, bool KV8, int NWV, int MODE>
 __global__ __launch_bounds__(64 * NWV) __attribute__((amdgpu_waves_per_eu(2, 2)))  // 256 registers: two waves per SIMD
 void prefill_attn_kernel(const PrefillParams p) {
+  static_assert(MODE == 0 || !KV8, "e4m3 rows always fit fp16");
+  constexpr bool VB16 = MODE == 1;
   __shared__ __attribute__((aligned(16))) unsigned short Ks[kBKV][kPRowK];  // bf16, rows in k_tile_row order
   __shared__ __attribute__((aligned(16))) unsigned short Vs[kBKV][kPRowV];  // fp16 (bf16 for a tile fp16 cannot hold)
   __shared__ __attribute__((aligned(16))) unsigned int vvote[8];            // per wave: what its V slice holds
@@ -189,6 +196,10 @@ void prefill_attn_kernel(const PrefillParams p) {
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int n = lane & 15, g = lane >> 4;
+  // first output element of this workgroup's row tile (row row0, first head of the KV head's group)
+  unsigned short *const marker =
+      p.out + (static_cast<int64_t>(q_begin + row0) * p.num_q_heads + static_cast<int64_t>(h) * group) * kPDh;
+  if (MODE == 1 && *marker != kRedoMarker) return;   // workgroup uniform
 
   // units of this lane: u = wave*CT*16 + c*16 + n -> (row, head)
   int urow[CT];
@@ -267,9 +278,9 @@ void prefill_attn_kernel(const PrefillParams p) {
     }
   };
   // What this wave's slice of the V tile in vreg holds: bit 0 some |v| >= 65536, bit 1 some |v| >= 2^-9,
-  // bit 2 anything but zeros, bit 3 some |v| >= 2^112.  (e4m3 rows always fit fp16.)
+  // bit 2 anything but zeros.
   auto vote_tile = [&]() __attribute__((always_inline)) {
-    if constexpr (!KV8) {
+    if constexpr (!KV8 && MODE == 0) {
       ushortx2 mx = ushortx2{0, 0};
 #pragma unroll
       for (int i = 0; i < kPasses; ++i) {
@@ -281,24 +292,23 @@ void prefill_attn_kernel(const PrefillParams p) {
       const unsigned int m = mx[0] > mx[1] ? mx[0] : mx[1];
       const unsigned int bits = (__builtin_amdgcn_ballot_w64(m >= kVBigBits) ? 1u : 0u) |
                                 (__builtin_amdgcn_ballot_w64(m >= kVDecentBits) ? 2u : 0u) |
-                                (__builtin_amdgcn_ballot_w64(m != 0u) ? 4u : 0u) |
-                                (__builtin_amdgcn_ballot_w64(m >= kVHugeBits) ? 8u : 0u);
+                                (__builtin_amdgcn_ballot_w64(m != 0u) ? 4u : 0u);
       if (lane == 0) vvote[wave] = bits;
     }
   };
-  // After the barrier that follows vote_tile(): the OR of the waves' votes (workgroup uniform)
-  auto tile_votes = [&]() __attribute__((always_inline)) -> unsigned int {
-    if constexpr (KV8) return 0u;
+  // After the barrier that follows vote_tile(): true when fp16 cannot hold the tile (workgroup uniform)
+  auto tile_needs_bf16 = [&]() __attribute__((always_inline)) -> bool {
+    if constexpr (KV8 || MODE == 1) return false;
     unsigned int any = 0;
 #pragma unroll
     for (int w = 0; w < NWV; w += 4) {
       const uint4 t = *reinterpret_cast<const uint4 *>(&vvote[w]);
       any |= t.x | t.y | t.z | t.w;
     }
-    return __builtin_amdgcn_readfirstlane(any);
+    any = __builtin_amdgcn_readfirstlane(any);
+    return (any & 1u) || ((any & 6u) == 4u);
   };
-  auto votes_need_bf16 = [](unsigned int any) { return (any & 1u) || ((any & 6u) == 4u); };
-  auto store_tile = [&](bool v_as_bf16) __attribute__((always_inline)) {
+  auto store_tile = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int i = 0; i < kPasses; ++i) {
       const int t = i * kRowsPerPass + trow;
@@ -314,7 +324,7 @@ void prefill_attn_kernel(const PrefillParams p) {
         *reinterpret_cast<uint4 *>(&Vs[t][64 + ch * 8]) = hi;
       } else {
         *reinterpret_cast<uint4 *>(&Ks[kr][ch * 8]) = kreg[i];
-        if (v_as_bf16)
+        if constexpr (VB16)
           *reinterpret_cast<uint4 *>(&Vs[t][ch * 8]) = vreg[i];
         else
           *reinterpret_cast<uint4 *>(&Vs[t][ch * 8]) =
@@ -337,25 +347,16 @@ void prefill_attn_kernel(const PrefillParams p) {
   load_tile(0);
   vote_tile();
   lds_barrier();
-  unsigned int votes = tile_votes();
-  float pshift = kPShift;            // P is carried as 2^pshift p: 15, or 0 once a tile with huge values was met
-  bool v_bf16 = votes_need_bf16(votes);   // of the tile in LDS
-  bool v_huge = (votes & 8u) != 0;
-  store_tile(v_bf16);
+  if (tile_needs_bf16()) {   // workgroup uniform
+    if (tid == 0) *marker = kRedoMarker;
+    return;
+  }
+  constexpr float pshift = VB16 ? 0.f : kPShift;   // P is carried as 2^pshift p
+  store_tile();
   lds_barrier();
   for (int kv0 = 0; kv0 < kv_end; kv0 += kBKV) {
     const bool more = kv0 + kBKV < kv_end;
     if (more) load_tile(kv0 + kBKV);
-    if (!KV8 && v_huge && pshift != 0.f) {  // workgroup uniform, at most once per workgroup
-      const float back = 0x1p-15f;
-#pragma unroll
-      for (int c = 0; c < CT; ++c) {
-        l_run[c] *= back;
-        rescale16(acc[c], 0, back);
-        rescale16(acc[c], 4, back);
-      }
-      pshift = 0.f;
-    }
     // tiles that end at or before the first row's limit and inside lk need no mask
     const bool need_mask = (kv0 + kBKV - 1 > shift + row0) || (kv0 + kBKV > lk);
 #pragma unroll
@@ -413,7 +414,7 @@ void prefill_attn_kernel(const PrefillParams p) {
         for (int j = 0; j < 8; ++j)  // 2^15 p = 2^(s * scale - m + 15): at most 2^15; a flushed denormal result is an exact 0 weight
           pv[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(sv[j], scale_log2, shift_m));
         const float psum = ((pv[0] + pv[1]) + (pv[2] + pv[3])) + ((pv[4] + pv[5]) + (pv[6] + pv[7]));
-        if (!KV8 && v_bf16) {  // workgroup uniform
+        if constexpr (VB16) {
           unsigned int hi[4], lo[4];
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
@@ -443,7 +444,7 @@ void prefill_attn_kernel(const PrefillParams p) {
         const shortx4 v1 = lds_read_tr16(&Vs[vt + 4][d * 16 + (n & 3) * 4]);
         const uint4 vraw = make_uint4(__builtin_bit_cast(uint2, v0).x, __builtin_bit_cast(uint2, v0).y,
                                       __builtin_bit_cast(uint2, v1).x, __builtin_bit_cast(uint2, v1).y);
-        if (!KV8 && v_bf16) {
+        if constexpr (VB16) {
           const bf16x8 vb = __builtin_bit_cast(bf16x8, vraw);
 #pragma unroll
           for (int c = 0; c < CT; ++c) {
@@ -461,10 +462,11 @@ void prefill_attn_kernel(const PrefillParams p) {
     if (more) vote_tile();   // of the tile that was loaded while this one was multiplied
     lds_barrier();
     if (more) {
-      votes = tile_votes();
-      v_huge = (votes & 8u) != 0;
-      v_bf16 = votes_need_bf16(votes) || v_huge || pshift == 0.f;
-      store_tile(v_bf16);
+      if (tile_needs_bf16()) {   // workgroup uniform
+        if (tid == 0) *marker = kRedoMarker;
+        return;
+      }
+      store_tile();
       lds_barrier();
     }
   }
@@ -574,11 +576,16 @@ extern "C" int tlf_varlen_prefill_attn(const void *q, int64_t q_stride, const vo
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (paged && kv_dtype == TLF_KV_FP8_E4M3) {
     // the K scale is a per-head constant of the scores: fold it in on the device side per head
-    if (nwv == 8) TLF_LAUNCH((prefill_attn_kernel<CT, true, 8>), grid, dim3(512), 0, s, p);
-    else TLF_LAUNCH((prefill_attn_kernel<CT, true, 4>), grid, dim3(256), 0, s, p);
+    if (nwv == 8) TLF_LAUNCH((prefill_attn_kernel<CT, true, 8, 0>), grid, dim3(512), 0, s, p);
+    else TLF_LAUNCH((prefill_attn_kernel<CT, true, 4, 0>), grid, dim3(256), 0, s, p);
   } else {
-    if (nwv == 8) TLF_LAUNCH((prefill_attn_kernel<CT, false, 8>), grid, dim3(512), 0, s, p);
-    else TLF_LAUNCH((prefill_attn_kernel<CT, false, 4>), grid, dim3(256), 0, s, p);
+    if (nwv == 8) TLF_LAUNCH((prefill_attn_kernel<CT, false, 8, 0>), grid, dim3(512), 0, s, p);
+    else TLF_LAUNCH((prefill_attn_kernel<CT, false, 4, 0>), grid, dim3(256), 0, s, p);
+    int rc = launch_status();
+    if (rc != TLF_OK) return rc;
+    // the row tiles that met a V tile outside fp16's range, again in bf16 (every other workgroup returns at once)
+    if (nwv == 8) TLF_LAUNCH((prefill_attn_kernel<CT, false, 8, 1>), grid, dim3(512), 0, s, p);
+    else TLF_LAUNCH((prefill_attn_kernel<CT, false, 4, 1>), grid, dim3(256), 0, s, p);
   }
   return launch_status();
 }
