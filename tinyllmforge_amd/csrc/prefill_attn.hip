@@ -547,15 +547,18 @@ extern "C" int tlf_varlen_prefill_attn(const void *q, int64_t q_stride, const vo
   p.block_size = block_size;
   p.num_cache_blocks = num_cache_blocks;
   p.scale_log2 = scale * kPLog2e;
-  constexpr int CT = 2;
-  // 4 waves (128 (row, head) units, two workgroups per CU) or 8 waves (256 units, one workgroup per CU: half
-  // the K/V staging per unit; measured 4-5 % faster on sequences of 4096 and 8192 tokens, no faster on 1024 and
-  // below, where the longer row tiles waste more of the diagonal); TLF_PREFILL_WAVES overrides for tuning
+  // Eight waves of 48 (row, head) units each (CT = 3 column tiles of 16: 384 units, one workgroup per CU), or four
+  // waves of 32 (CT = 2, two workgroups per CU).  Every wave reads the whole K and V tile out of LDS for its own
+  // units, so LDS bytes per MFMA fall as 1 / CT, and with two column tiles the LDS reads alone take as long as
+  // the MFMAs; three is what 256 registers hold.  Measured, 3 x 8 against 2 x 8 / 2 x 4: 16 x 1024 tokens
+  // 284 us against 297 (2 x 4), 4 x 4096 740 against 793, 2 x 8192 on e4m3 rows 2362 against 2579.
+  // TLF_PREFILL_WAVES=4 picks the four-wave form for tuning.
   static const int forced = [] {
     const char *e = getenv("TLF_PREFILL_WAVES");
-    return e && atoi(e) == 4 ? 4 : e && atoi(e) == 8 ? 8 : 0;
+    return e && atoi(e) == 4 ? 4 : 0;
   }();
-  const int nwv = forced ? forced : max_seqlen_q >= 2048 ? 8 : 4;
+  const int nwv = forced ? forced : 8;
+  const int ct = nwv == 8 ? 3 : 2;
   // An XCD walks its (sequence, KV head) pairs four at a time with the row tiles outermost, longest first: with
   // one pair after the other the last pair's long row tiles start when most slots are already idle (16 x 1024
   // tokens 304 -> 287 us, 28 x 560 190 -> 182, 4 x 4096 779 -> 757); four pairs' K/V rows (2 MB at 1024 tokens)
@@ -571,21 +574,21 @@ extern "C" int tlf_varlen_prefill_attn(const void *q, int64_t q_stride, const vo
     while (grp > 1 && (per_xcd < 1 || per_xcd % grp)) grp >>= 1;
     p.pair_group = grp;
   }
-  const int bq = (16 * nwv * CT) / group;
+  const int bq = (16 * nwv * ct) / group;
   const dim3 grid((max_seqlen_q + bq - 1) / bq, num_kv_heads, num_seqs);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (paged && kv_dtype == TLF_KV_FP8_E4M3) {
     // the K scale is a per-head constant of the scores: fold it in on the device side per head
-    if (nwv == 8) TLF_LAUNCH((prefill_attn_kernel<CT, true, 8, 0>), grid, dim3(512), 0, s, p);
-    else TLF_LAUNCH((prefill_attn_kernel<CT, true, 4, 0>), grid, dim3(256), 0, s, p);
+    if (nwv == 8) TLF_LAUNCH((prefill_attn_kernel<3, true, 8, 0>), grid, dim3(512), 0, s, p);
+    else TLF_LAUNCH((prefill_attn_kernel<2, true, 4, 0>), grid, dim3(256), 0, s, p);
   } else {
-    if (nwv == 8) TLF_LAUNCH((prefill_attn_kernel<CT, false, 8, 0>), grid, dim3(512), 0, s, p);
-    else TLF_LAUNCH((prefill_attn_kernel<CT, false, 4, 0>), grid, dim3(256), 0, s, p);
+    if (nwv == 8) TLF_LAUNCH((prefill_attn_kernel<3, false, 8, 0>), grid, dim3(512), 0, s, p);
+    else TLF_LAUNCH((prefill_attn_kernel<2, false, 4, 0>), grid, dim3(256), 0, s, p);
     int rc = launch_status();
     if (rc != TLF_OK) return rc;
     // the row tiles that met a V tile outside fp16's range, again in bf16 (every other workgroup returns at once)
-    if (nwv == 8) TLF_LAUNCH((prefill_attn_kernel<CT, false, 8, 1>), grid, dim3(512), 0, s, p);
-    else TLF_LAUNCH((prefill_attn_kernel<CT, false, 4, 1>), grid, dim3(256), 0, s, p);
+    if (nwv == 8) TLF_LAUNCH((prefill_attn_kernel<3, false, 8, 1>), grid, dim3(512), 0, s, p);
+    else TLF_LAUNCH((prefill_attn_kernel<2, false, 4, 1>), grid, dim3(256), 0, s, p);
   }
   return launch_status();
 }
