@@ -506,6 +506,10 @@ def bench_c5(args):
                cached_prompt_tokens=st["cached_prompt_tokens"],
                decode_byte_floor=decode_byte_floor(llm.config.hf_config, st, "w8a16", kv_itemsize=1),
                kv_blocks=llm.config.num_kvcache_blocks, kv_dtype="fp8_e4m3")
+    sat = llm.model_runner.kv_saturation()                      # after the timed region
+    res["kv_saturated_fraction"] = dict(k=round(sat["k_saturated"] / max(1, sat["entries"]), 8),
+                                        v=round(sat["v_saturated"] / max(1, sat["entries"]), 8),
+                                        k_worst=sat["k_worst"], v_worst=sat["v_worst"])
     llm.exit()
     return res
 

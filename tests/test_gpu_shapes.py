@@ -354,3 +354,40 @@ def test_32b_width_two_layers_fp8_kv_with_cached_prefix_against_the_oracle():
     finally:
         close(llm)
     assert m["hidden_l2"] <= 2 * WIDTH_TOL and m["row_l2"] <= 2 * WIDTH_TOL and m["ulps"] <= 4.0, m   # measured: 2.0 ... 3.0
+
+
+def test_e4m3_cache_saturation_is_counted_per_layer_and_head():
+    """An e4m3 cache clamps at +-448 x scale without an error; `ModelRunner.kv_saturation` counts the clamped
+    entries.  Planted codes are found where they were put; a run with an absurdly small K scale saturates K and
+    leaves V alone; a bf16 cache reports nothing."""
+    from tinyllmforge_amd import LLM, SamplingParams
+    cfg = width_config("qwen3-0.6b")
+    llm = LLM(cfg, max_model_len=1024, max_num_batched_tokens=2048, max_num_seqs=4, num_kvcache_blocks=6,
+              enforce_eager=True, seed=1, kv_cache_dtype="fp8_e4m3", kv_k_scale=1e-4, kv_v_scale=4.0)
+    try:
+        mr = llm.model_runner
+        assert mr.kv_saturation() == dict(entries=mr.kv_cache[0].numel(), k_saturated=0, v_saturated=0,
+                                          k_worst=None, v_worst=None)
+        with torch.inference_mode():           # the cache was allocated under inference mode
+            kv = mr.kv_cache.view(torch.uint8)
+            kv[0, 1, 2, 5:9, 3, :] = 0x7e      # K, layer 1, block 2, four rows of KV head 3: +448 x scale
+            kv[0, 0, 4, 0, 1, :7] = 0xfe       # K, layer 0: seven entries at -448 x scale
+            kv[1, 1, 0, 0, 0, 0] = 0x7d        # V: the largest code below saturation
+        got = mr.kv_saturation()
+        assert got["k_saturated"] == 4 * 128 + 7 and got["v_saturated"] == 0
+        assert got["k_worst"] == dict(layer=1, kv_head=3, saturated=4 * 128) and got["v_worst"] is None
+        assert mr.kv_saturation(block_ids=[4])["k_saturated"] == 7
+        with torch.inference_mode():
+            mr.kv_cache.zero_()
+        llm.generate(random_prompts((300,), seed=3, vocab=10000), SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))
+        got = mr.kv_saturation()
+        # k after q/k-norm is of order 1: with a scale of 1e-4 almost every written K entry clamps; |v| << 448 x 4
+        assert got["k_saturated"] > 0.9 * 2 * 303 * cfg["num_key_value_heads"] * 128 and got["v_saturated"] == 0, got
+    finally:
+        close(llm)
+    llm = LLM(cfg, max_model_len=1024, max_num_batched_tokens=2048, max_num_seqs=4, num_kvcache_blocks=6,
+              enforce_eager=True, seed=1)
+    try:
+        assert llm.model_runner.kv_saturation()["entries"] == 0
+    finally:
+        close(llm)

@@ -126,6 +126,30 @@ class ModelRunner:
                     module.v_scale = self._kv_scale(cfg.kv_v_scale, layer_id)
                 layer_id += 1
 
+    @torch.inference_mode()
+    def kv_saturation(self, block_ids=None) -> dict:
+        """How many entries of an e4m3 KV cache sit at the format's largest magnitude (|code| = 0x7e, i.e.
+        +-448 x scale): the store clamps there, so a scale too small for a layer's keys or values shows up as
+        saturated entries, not as an error.  Counted over ``block_ids`` (default: every block; unwritten rows
+        are zeros and count as entries).  Returns totals and the worst (layer, KV head) for K and for V; a bf16
+        cache has nothing to saturate and returns zeros."""
+        out = dict(entries=0, k_saturated=0, v_saturated=0, k_worst=None, v_worst=None)
+        if self.kv_cache is None or self.kv_dtype == torch.bfloat16:
+            return out
+        kv = self.kv_cache.view(torch.uint8)                       # [2, L, nblk, block, Hkv, Dh]
+        if block_ids is not None:
+            kv = kv[:, :, torch.as_tensor(sorted(set(block_ids)), dtype=torch.long, device=kv.device)]
+        out["entries"] = int(kv[0].numel())
+        for which, name in ((0, "k"), (1, "v")):
+            per = torch.zeros(kv.shape[1], kv.shape[4], dtype=torch.int64, device=kv.device)
+            for layer in range(kv.shape[1]):                        # one layer at a time: the mask is a byte per entry
+                per[layer] = ((kv[which, layer] & 0x7f) == 0x7e).sum(dim=(0, 1, 3))
+            out[name + "_saturated"] = int(per.sum())
+            if out[name + "_saturated"]:
+                layer, head = divmod(int(per.argmax()), kv.shape[4])
+                out[name + "_worst"] = dict(layer=layer, kv_head=head, saturated=int(per[layer, head]))
+        return out
+
     def _kv_scale(self, spec, layer_id: int) -> torch.Tensor:
         """fp32 ``[Hkv]`` from a float (every head), ``[Hkv]`` values (every layer) or ``[L][Hkv]`` values."""
         hkv = self.config.hf_config.num_key_value_heads
