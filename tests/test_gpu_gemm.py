@@ -146,6 +146,33 @@ def test_w8a16_config3_cell(M, name):
         assert (got.float().cpu() - want.float()).abs().max().item() <= 2e-2 * max(1.0, want.float().abs().max().item() / 4)
 
 
+# The Qwen3-32B projections at 1 ... 12 tokens: on matrices this large the planner hands batches below 13 tokens to
+# the W-streaming kernel instead of the skinny one (gate_up and down at every count, qkv and o_proj from 8 on).
+SHAPES_32B = {"qkv_32b": (10240, 5120), "o_proj_32b": (5120, 8192), "gate_up_32b": (51200, 5120), "down_32b": (5120, 25600)}
+
+
+@pytest.mark.parametrize("name", list(SHAPES_32B))
+def test_w8a16_32b_shapes_below_13_tokens_exact_on_integer_data(name):
+    import ctypes
+    from tinyllmforge_amd import _lib, ops as P
+    N, K = SHAPES_32B[name]
+    wq = torch.randint(-127, 128, (N, K), generator=g(N + K), dtype=torch.int32).to(torch.int8).to(DEV)
+    packed = P.pack_w8(wq)
+    scale = torch.full((N,), 2.0 ** -12, device=DEV)
+    kinds = set()
+    for M in (1, 3, 4, 7, 8, 12):
+        plan = (ctypes.c_int32 * 8)()
+        assert _lib.load().tlf_gemm_plan(M, N, K, 1, plan) == 0
+        kinds.add("skinny" if plan[0] == 0 else "w-streaming")
+        x = torch.randint(-2, 3, (M, K), generator=g(M), dtype=torch.int32).to(BF).to(DEV)
+        got = P.w8a16_linear(x, packed, scale)
+        ref = ((x.double() @ wq.double().t()) * 2.0 ** -12).to(BF)
+        assert torch.equal(got.view(torch.int16), ref.view(torch.int16)), (M, list(plan))
+    assert "w-streaming" in kinds, kinds
+    if name in ("qkv_32b", "o_proj_32b"):
+        assert "skinny" in kinds, kinds
+
+
 @pytest.mark.parametrize("M", [4, 48, 256, 600])
 def test_w8a16_weight_larger_than_2_gib(M):
     """An int8 weight of 2.06 GiB (270,336 x 8192): byte offsets into the tile-ordered weight pass 2^31 in the

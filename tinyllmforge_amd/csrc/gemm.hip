@@ -961,6 +961,7 @@ struct GemmTuning {
   int skinny_pipe_m = -1;  // forced token limit of the skinny kernel's two-batch pipeline
   int group_n = 0;
   int ws_min_m = 13, ws_max_m = 224;  // token range of the W-streaming kernel (int8 weights)
+  bool ws_range_set = false;          // the range came from TLF_GEMM_WSTREAM_M: taken literally
   int ws_splits = 0;                               // forced split of K for it
   int ws_kg = 0;                                   // forced K parts per workgroup (1 or 2)
   bool ws_force = false;                           // take it for every shape in its token range
@@ -992,6 +993,7 @@ inline const GemmTuning &gemm_tuning() {
       if (sscanf(e, "%d,%d", &lo, &hi) == 2) {
         g.ws_min_m = lo < 1 ? 1 : lo;
         g.ws_max_m = hi > 224 ? 224 : hi;  // seven token tiles of 32 is the tallest instance
+        g.ws_range_set = true;
       }
     }
     if (const char *e = getenv("TLF_GEMM_WSTREAM_SPLITS")) g.ws_splits = atoi(e) > 0 ? atoi(e) : 0;
@@ -1060,7 +1062,20 @@ struct GemmPlan {
 // when N alone fills the machine.
 inline bool plan_wstream(int M, int N, int K, int act, GemmPlan &g) {
   const GemmTuning &t = gemm_tuning();
-  if (t.has_plan || M < t.ws_min_m || M > t.ws_max_m || M < 1 || act == 2) return false;
+  if (t.has_plan || M > t.ws_max_m || M < 1 || act == 2) return false;
+  if (M < t.ws_min_m) {
+    // Below 13 tokens the skinny kernel runs, except on big matrices, where one workgroup per 96 or 128 channels
+    // streaming its rows beats the skinny kernel's many small workgroups.  Cold weights, us, W-streaming / skinny
+    // at 1 / 4 / 8 / 12 tokens: 51200 x 5120 44.8 / 45.1 / 45.8 / 46.7 against 53.6 / 55.0 / 49.8 / 51.5;
+    // 5120 x 25600 27.5 / 26.6 / 26.7 / 26.8 against 34.5 / 35.5 / 42.7 / 49.0; 10240 x 5120 15.5 / 14.4 / 15.0 / 14.5
+    // against 14.5 / 14.8 / 15.8 / 18.3; 5120 x 8192 13.6 / 13.5 / 13.5 / 13.9 against 12.5 / 13.0 / 15.4 / 17.6;
+    // 24576 x 4096 18.8 / 18.8 / 18.9 / 18.8 against 18.6 / 18.4 / 19.4 / 20.5; but 4096 x 12288 16.4 / 15.3 / 15.6 / 15.7
+    // against 11.4 / 11.2 / 12.8 / 16.6 and 6144 x 4096 10.0 against 8.2 ... 10.3.
+    const int64_t nk = static_cast<int64_t>(N) * K;
+    const bool big = nk >= 120000000;
+    const bool mid = M >= 8 && nk >= 40000000 && N >= 5120;
+    if (t.ws_range_set || !(big || mid)) return false;
+  }
   if (M > 128 && !(N >= 256 * 96)) return false;  // 129 ... 224 tokens: 96-channel workgroups on a wide N only (below)
   // 13 ... 16 tokens, cold weights, W-streaming / skinny kernel at 16 tokens: qkv 10.5 / 11.8 us, gate_up 20.1 / 22.2,
   // down 16.5 / 18.1, but o_proj (N = 4096, K = 4096: 43 workgroups x 4 splits) 9.3 / 7.8
