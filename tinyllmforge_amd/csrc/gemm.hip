@@ -1093,6 +1093,9 @@ inline bool plan_wstream(int M, int N, int K, int act, GemmPlan &g) {
   if (M > 128) cols = 3;
   if (t.ws_cols == 3 || t.ws_cols == 4) cols = t.ws_cols;
   const int n_wg = (N + cols * 32 - 1) / (cols * 32);
+  // ... and only when those workgroups fill whole rounds of the CUs: 51200 channels are 534 workgroups (2.1 rounds), and
+  // the tiled plans win there (160 / 192 / 224 tokens 114.3 / 130.4 / 146.4 us against 122.6 / 143.1 / 164.3)
+  if (M > 128 && !t.ws_force && fill(n_wg) < 0.9) return false;
   int splits = 1;
   // Measured against the tiled plans on the Qwen3-8B projections with cold weights: a wide N (gate_up)
   // wins at every size up to 128 tokens (24 / 28 / 37 us at 32 / 64 / 128 tokens against 36 / 38 / 43);
@@ -1101,7 +1104,11 @@ inline bool plan_wstream(int M, int N, int K, int act, GemmPlan &g) {
   // 80 tokens (qkv 10.5 / 11.2 / 14.4 / 16.2 us at 17 / 32 / 64 / 80 tokens against 14.3 / 14.7 / 16.3 / 17.3 for
   // the tiled plans, o_proj 9.5 / 9.7 / 12.1 / 14.2 against 13.1 / 13.5 / 14.9 / 14.7) and, with a long K (down
   // projection), up to 32 (16.0 / 16.9 at 17 / 32 against 25.8 / 25.9); above that the tiled plans are faster.
-  if (!t.ws_force && narrow && M > (ktiles >= 128 ? 32 : 80)) return false;
+  // The bigger narrow matrices of the Qwen3-32B shape keep winning up to 128 tokens (cold weights, us, W-streaming /
+  // tiled at 64 / 96 / 128 tokens: 10240 x 5120 20.0 / 24.3 / 28.2 against 20.0 / 31.3 / 35.8; 5120 x 8192 18.0 / 21.6 /
+  // 25.1 against 23.2 / 26.2 / 31.0; 5120 x 25600 36.7 / 44.3 / 49.8 against 48.6 / 56.6 / 65.8).
+  const bool big_narrow = static_cast<int64_t>(N) * K >= 40000000 && N >= 5120 && M <= 128;
+  if (!t.ws_force && narrow && M > (ktiles >= 128 ? 32 : 80) && !big_narrow) return false;
   if (act) {
     if (narrow) return false;
   } else {
