@@ -1161,7 +1161,22 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
   //  - wide N (gate_up) from 193 to 256 tokens: 256 x 128 tile with eight waves (256 tokens: 60.8 against 71.2).
   const bool tall_long_k = w8 && n128 < 128 && ktiles > 64 && M > 32 && M <= 208;
   const bool mid_k64 = w8 && n128 < 128 && n128 >= 48 && ktiles <= 64 && ktiles % 4 == 0 && M > 160 && M <= 256;
-  if (tall_long_k || (mid_k64 && M <= 224)) {
+  // The narrow projections of the Qwen3-32B shape (10240 x 5120, 5120 x 8192, 5120 x 25600) above the W-streaming
+  // kernel's 128 tokens, from a sweep of 16 plans on cold weights (us, this plan / the rules below): 192 tokens
+  // 128 x 64 tiles with K split 2 (4 from K = 8192 on) 40.4 / 33.3 / 81.3 against 48.4 / 42.3 / 88.9; 256 tokens 256 x 128
+  // tiles, same splits, 45.2 / 37.4 / 88.8 against 52.8 / 43.9 / 97.8.  (The Qwen3-8B shapes keep the rules below: the
+  // same sweep found nothing faster for them.)
+  const bool big_narrow = w8 && n128 < 128 && N >= 5120 && static_cast<int64_t>(N) * K >= 40000000;
+  bool measured_splits = false;   // the split came out of a sweep: the long-K adjustment below leaves it alone
+  if (big_narrow && M > 128 && M <= 256) {
+    if (M <= 192) {
+      g.bn = 128; g.bm = 64; g.stages = 4; g.occ = 3; g.wn = 4;
+    } else {
+      g.bn = 256; g.bm = 128; g.stages = 3; g.occ = 2; g.wn = 8;
+    }
+    splits = K >= 8192 ? 4 : 2;
+    measured_splits = true;
+  } else if (tall_long_k || (mid_k64 && M <= 224)) {
     g.bn = 128; g.bm = M <= 64 ? 64 : (M + 31) / 32 * 32; g.wn = 4;
     g.stages = g.bm == 64 ? 4 : 3; g.occ = g.bm == 64 ? 3 : 2;
     splits = tall_long_k ? 8 : 4;
@@ -1239,7 +1254,7 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
     g.bn = 256; g.bm = 128; g.stages = 3; g.occ = 1;
   }
   // a long K wants a split of its own: no workgroup walks more than ~48 K-tiles when splitting
-  if (splits > 1 && splits < pow2_floor(ktiles / 48)) splits = pow2_floor(ktiles / 48);
+  if (!measured_splits && splits > 1 && splits < pow2_floor(ktiles / 48)) splits = pow2_floor(ktiles / 48);
   if (splits > max_split) splits = max_split;
   if (splits > 16) splits = 16;
   if (splits < 1) splits = 1;
