@@ -173,6 +173,19 @@ def test_w8a16_32b_shapes_below_13_tokens_exact_on_integer_data(name):
         assert "skinny" in kinds, kinds
 
 
+@pytest.mark.parametrize("M,N,K", [(6000, 5120, 8192), (16384, 6144, 4096), (5000, 10240, 5120), (4352, 4096, 4096)])
+def test_w8a16_many_tile_rows_exact_on_integer_data(M, N, K):
+    """From 16 tile rows on an XCD may own tile rows instead of tile columns (whichever shares out more evenly over
+    the 8 XCDs): ragged last row tile, 20 / 24 / 40 / 16 tile columns, 24 / 64 / 20 / 17 tile rows."""
+    from tinyllmforge_amd import ops as P
+    x = torch.randint(-2, 3, (M, K), generator=g(M), dtype=torch.int32).to(BF).to(DEV)
+    wq = torch.randint(-127, 128, (N, K), generator=g(N + K), dtype=torch.int32).to(torch.int8).to(DEV)
+    got = P.w8a16_linear(x, P.pack_w8(wq), torch.full((N,), 2.0 ** -12, device=DEV))
+    for m0 in range(0, M, 2048):
+        ref = ((x[m0:m0 + 2048].double() @ wq.double().t()) * 2.0 ** -12).to(BF)
+        assert torch.equal(got[m0:m0 + 2048].view(torch.int16), ref.view(torch.int16)), m0
+
+
 @pytest.mark.parametrize("M", [4, 48, 256, 600])
 def test_w8a16_weight_larger_than_2_gib(M):
     """An int8 weight of 2.06 GiB (270,336 x 8192): byte offsets into the tile-ordered weight pass 2^31 in the

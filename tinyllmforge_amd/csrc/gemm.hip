@@ -199,13 +199,21 @@ void gemm_dlds_kernel(const GemmParams p) {
   // groups of group_n: inside a group the M-tiles are walked with the group's columns innermost,
   // so the ~32 workgroups resident on an XCD form a patch of (32 / group_n) x panels times
   // group_n W panels and the XCD's L2 fetches each panel once per K-tile.
+  // With many more tokens than channels the roles are swapped (xcd_rows): XCD b % 8 owns the M-tile rows
+  // mt = 8 r + xcd and walks all columns, group_n rows at a time with the rows innermost, so each XCD's L2 holds an
+  // eighth of x and streams W, instead of holding an eighth of W and streaming all of x (at 16384 tokens x is 6 x the
+  // bytes of a 5120 x 8192 weight), and 20 tile columns, which do not divide by 8, no longer leave four XCDs with
+  // half as much to do again as the other four.
   const int xcd = blockIdx.x & 7;
   const int local = blockIdx.x >> 3;
-  const int per_group = p.group_n * p.m_tiles;
+  const int walked = p.xcd_rows ? p.n_tiles : p.m_tiles;     // tiles along the dimension the XCD walks in full
+  const int per_group = p.group_n * walked;
   const int within = local % per_group;
-  const int mt = within / p.group_n;
-  const int nt = ((local / per_group) * p.group_n + within % p.group_n) * 8 + xcd;
-  if (nt >= p.n_tiles) return;
+  const int across = within / p.group_n;
+  const int owned = ((local / per_group) * p.group_n + within % p.group_n) * 8 + xcd;
+  const int mt = p.xcd_rows ? owned : across;
+  const int nt = p.xcd_rows ? across : owned;
+  if (nt >= p.n_tiles || mt >= p.m_tiles) return;
   const int n0 = nt * BN, m0 = mt * BM;
   const int split = blockIdx.y;
   const int tid = threadIdx.x;
@@ -948,6 +956,7 @@ void skinny_gemm_kernel(const GemmParams p) {
 //   TLF_GEMM_SKINNY_MAX_M   hand-over point between the skinny and the tiled kernel (0 ... 64)
 //   TLF_GEMM_SKINNY_TN      16-channel tiles per skinny workgroup (1, 2 or 4)
 //   TLF_GEMM_GROUP_N        N-tile columns per XCD patch
+//   TLF_GEMM_XCD_ROWS=0|1   an XCD owns tile columns | tile rows (the planner picks by tile counts)
 //   TLF_GEMM_WSTREAM_M="lo,hi"  token range served by the W-streaming kernel ("0,0": never)
 //   TLF_GEMM_WSTREAM_SPLITS     its split of K across workgroups
 //   TLF_GEMM_WSTREAM_KG         its K parts inside a workgroup (1 or 2)
@@ -960,6 +969,7 @@ struct GemmTuning {
   int skinny_tn = 0;
   int skinny_pipe_m = -1;  // forced token limit of the skinny kernel's two-batch pipeline
   int group_n = 0;
+  int xcd_rows = -1;   // TLF_GEMM_XCD_ROWS: -1 planner's choice
   int ws_min_m = 13, ws_max_m = 224;  // token range of the W-streaming kernel (int8 weights)
   bool ws_range_set = false;          // the range came from TLF_GEMM_WSTREAM_M: taken literally
   int ws_splits = 0;                               // forced split of K for it
@@ -988,6 +998,7 @@ inline const GemmTuning &gemm_tuning() {
     }
     if (const char *e = getenv("TLF_GEMM_SKINNY_PIPE_M")) g.skinny_pipe_m = atoi(e);
     if (const char *e = getenv("TLF_GEMM_GROUP_N")) g.group_n = atoi(e) > 0 ? atoi(e) : 1;
+    if (const char *e = getenv("TLF_GEMM_XCD_ROWS")) g.xcd_rows = atoi(e) != 0;
     if (const char *e = getenv("TLF_GEMM_WSTREAM_M")) {
       int lo = 0, hi = 0;
       if (sscanf(e, "%d,%d", &lo, &hi) == 2) {
@@ -1302,10 +1313,11 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   p.act = act;
   p.amax = nullptr;
   p.amax_parts = 0;
+  p.xcd_rows = 0;
   GemmPlan g;
   const bool wstream = W8 && plan_wstream(M, N, K, act, g);
   if (M <= skinny_max_m() && !wstream) {
-    p.k_per_split = K; p.splits = 1; p.m_tiles = 1; p.n_tiles = 1; p.group_n = 1;
+    p.k_per_split = K; p.splits = 1; p.m_tiles = 1; p.n_tiles = 1; p.group_n = 1; p.xcd_rows = 0;
     if (dry) {
       const int32_t skinny[8] = {0, 0, 0, 0, 1, 1, K, 1};  // tile 0 x 0 = the skinny kernel
       for (int i = 0; i < 8; ++i) plan_out[i] = skinny[i];
@@ -1349,14 +1361,24 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   }
   // XCD patch: group as many N-tile columns as divide this XCD's share evenly (up to 4), once
   // there are enough M-tiles for the patch to matter
+  // An XCD owns tile rows instead of tile columns (see the kernel) from 16 tile rows on, unless the columns share out
+  // over the 8 XCDs more evenly than the rows.  Measured at 8192 / 16384 tokens, us, rows / columns: 5120 x 8192
+  // 569 / 644 and 1063 / 1288, 5120 x 25600 1782 / 1967 and 3311 / 3920, 51200 x 5120 3367 / 3529 and 6744 / 7052,
+  // 10240 x 5120 676 / 706 and 1344 / 1404; the Qwen3-8B shapes 1-2 % faster; at 2048 tokens (8 tile rows) no gain.
+  // TLF_GEMM_XCD_ROWS = 0 / 1 forces the choice for tuning.
   {
-    const int cols = (p.n_tiles + 7) / 8;
-    if (p.m_tiles >= 8) g.group_n = cols % 4 == 0 ? 4 : cols % 3 == 0 ? 3 : cols % 2 == 0 ? 2 : 1;
+    auto padded = [](int tiles) { return static_cast<double>((tiles + 7) / 8 * 8) / tiles; };
+    p.xcd_rows = p.m_tiles >= 16 && padded(p.m_tiles) <= padded(p.n_tiles);
+  }
+  if (gemm_tuning().xcd_rows >= 0) p.xcd_rows = gemm_tuning().xcd_rows && p.m_tiles >= 8;
+  {
+    const int owned = ((p.xcd_rows ? p.m_tiles : p.n_tiles) + 7) / 8;
+    if ((p.xcd_rows ? p.n_tiles : p.m_tiles) >= 8) g.group_n = owned % 4 == 0 ? 4 : owned % 3 == 0 ? 3 : owned % 2 == 0 ? 2 : 1;
     if (gemm_tuning().group_n) g.group_n = gemm_tuning().group_n;
   }
   p.group_n = g.group_n;
-  const int cols_per_xcd = ((p.n_tiles + 7) / 8 + g.group_n - 1) / g.group_n * g.group_n;
-  const dim3 grid(cols_per_xcd * 8 * p.m_tiles, g.splits);
+  const int owned_per_xcd = (((p.xcd_rows ? p.m_tiles : p.n_tiles) + 7) / 8 + g.group_n - 1) / g.group_n * g.group_n;
+  const dim3 grid(owned_per_xcd * 8 * (p.xcd_rows ? p.n_tiles : p.m_tiles), g.splits);
   bool launched = false;
   if constexpr (W8) {
     if (g.wstream) {

@@ -29,7 +29,8 @@ struct GemmParams {
   int32_t k_per_split;
   int32_t splits;
   int32_t m_tiles, n_tiles;
-  int32_t group_n;  // N-tile columns walked together by one XCD
+  int32_t group_n;  // N-tile columns (xcd_rows: M-tile rows) walked together by one XCD
+  int32_t xcd_rows; // 1: an XCD owns M-tile rows 8 c + xcd and walks all N-tile columns; 0: it owns N-tile columns
   int32_t act;      // 1: SiLU-and-mul epilogue over interleaved gate/up channels, y is [M, N/2]
                     // 2: greedy-sample epilogue, nothing but argmax keys [M, amax_parts] is stored
   unsigned long long *amax;
