@@ -1368,7 +1368,7 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   // TLF_GEMM_XCD_ROWS = 0 / 1 forces the choice for tuning.
   {
     auto padded = [](int tiles) { return static_cast<double>((tiles + 7) / 8 * 8) / tiles; };
-    p.xcd_rows = p.m_tiles >= 16 && padded(p.m_tiles) <= padded(p.n_tiles);
+    p.xcd_rows = p.m_tiles >= 16 && padded(p.m_tiles) <= padded(p.n_tiles) * 1.04;   // rows also win a tie by 4 % (less traffic)
   }
   if (gemm_tuning().xcd_rows >= 0) p.xcd_rows = gemm_tuning().xcd_rows && p.m_tiles >= 8;
   {
