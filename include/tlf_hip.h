@@ -385,10 +385,14 @@ int tlf_paged_decode_attn(const void *q, int64_t q_stride,
  *     tlf_paged_decode_attn) and EVERY sequence reads its keys from them
  *     (layers/attention.py:99-100).
  * out: bf16 [total_q, Hq*Dh] contiguous.  max_seqlen_q bounds the grid.
- * fp32 softmax and accumulation.  The P.V product runs in fp16: P (in [0, 1], 11 significant bits;
- * flash-attn rounds it to one bf16, 8 bits) and V, which is converted to fp16 when its tile is staged
- * - exact for e4m3 rows, exact for bf16 rows between 6.1e-5 and 65504 in magnitude; smaller values keep
- * 2^-24 absolute resolution, larger ones saturate at 65504.
+ * fp32 softmax and accumulation.  The P.V product runs in fp16: P with 11 significant bits (flash-attn rounds
+ * it to one bf16, 8 bits), carried as 2^15 p so that weights down to 2^-29 of the row maximum are normal fp16
+ * numbers (the factor cancels in O / l), and V converted to fp16 when its tile is staged (exact for e4m3 rows).
+ * The input domain stays that of bf16 operands: a 64-token tile of bf16 V rows that fp16 cannot hold (some
+ * |v| >= 65536, or no element as large as 2^-9) makes the workgroup leave a marker in its first output element,
+ * and a second launch inside this call recomputes exactly those row tiles with both products in bf16 (P as a
+ * bf16 hi + lo pair).  So the call is two launches for bf16 rows and one for e4m3 rows; out is complete when
+ * the call's work on the stream is.
  * Dh == 128, Hq % Hkv == 0.
  */
 int tlf_varlen_prefill_attn(const void *q, int64_t q_stride,
