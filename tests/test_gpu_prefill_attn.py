@@ -258,3 +258,44 @@ def test_prefill_one_dominant_key_and_thousands_of_faint_ones(fp8):
     rows = [(0, 8191), (0, 8000), (0, 6001), (0, 4096), (0, 1500), (0, 300), (0, 0)]
     rel = _sampled_rows_check(q, kc, vc, cq, ck, bt, scale, got, rows, **okw)
     print(f"PREFILL_ERR sink fp8={fp8}: rel l2 {rel:.2e}, faint keys carry {w[1:].sum().item() / w.sum().item():.2f} of the mass")
+
+
+def test_prefill_two_launches_replay_in_a_hipgraph():
+    """A call on bf16 rows is two launches (the fp16-product kernel, then the bf16 pass over the row tiles that left
+    a marker).  Captured in a hipGraph and replayed several times, with eager work and synchronisations between the
+    replays and a fresh (garbage) output buffer content before each, every replay must equal the eager result bit for
+    bit - on inputs where some row tiles take the bf16 pass and some do not."""
+    from tinyllmforge_amd import ops as P
+    Hq, Hkv, Dh = 32, 8, 128
+    lens = [700, 130]
+    S = sum(lens)
+    ge = g(77)
+    q = torch.randn(S, Hq, Dh, generator=ge).to(BF).to(DEV)
+    k = torch.randn(S, Hkv, Dh, generator=ge).to(BF).to(DEV)
+    v = torch.randn(S, Hkv, Dh, generator=ge)
+    v[400, 3] *= 1e5                 # one head of one row beyond fp16: the row tiles that see it are redone in bf16
+    v[100:300] *= 1e-6               # whole tiles below 2^-9
+    v = v.to(BF).to(DEV)
+    c = cu(lens).to(DEV)
+    scale = Dh ** -0.5
+    eager = P.varlen_prefill_attention(q, k, v, c, c, max(lens), scale).clone()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        P.varlen_prefill_attention(q, k, v, c, c, max(lens), scale)      # warm-up on the capture stream
+        with torch.cuda.graph(graph, stream=side):
+            out = P.varlen_prefill_attention(q, k, v, c, c, max(lens), scale)
+    torch.cuda.synchronize()
+    for i in range(5):
+        if i == 4:
+            out.view(torch.int16).fill_(-91)             # 0xffa5 everywhere: the kernel's own marker pattern as stale content
+        else:
+            out.fill_(float("nan") if i % 2 else 7.0)    # stale contents, including NaN patterns, must not matter
+        junk = torch.randn(1 << 20, device=DEV).sum()    # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.view(torch.int16), eager.view(torch.int16)), f"replay {i}"
+        assert torch.isfinite(junk)
