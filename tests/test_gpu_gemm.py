@@ -231,7 +231,8 @@ def test_bf16_gemm(M, N, K):
 
 @pytest.mark.parametrize("M,N,K", [(1, 6144, 1024), (16, 2048, 4096), (130, 24576, 1024), (300, 6144, 2048),
                                    (2048, 4096, 512), (70, 16384, 192), (33, 272, 64), (2100, 24576, 128),
-                                   (300, 2064, 128), (150, 24592, 256), (20, 24592, 128)])   # N % 32 == 16
+                                   (300, 2064, 128), (150, 24592, 256), (20, 24592, 128),   # N % 32 == 16
+                                   (8, 24576, 4096), (12, 24576, 4096), (1, 51200, 5120), (4, 51200, 5120)])  # W-streaming below 13 tokens
 def test_w8a16_gemm_fused_silu_mul_equals_the_two_kernels(M, N, K):
     """gate_up projection + SiLU-and-mul in one kernel (interleaved weight rows) is bit-identical to the
     plain GEMM on the same weight followed by the activation kernel, and within tolerance of the oracle."""
