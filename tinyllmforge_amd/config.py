@@ -84,6 +84,11 @@ class Config:
     kv_v_scale: Any = 1.0 / 16
     seed: int = 0                           # random-init seed when no weights are given
     decode_position_quirk: bool = True      # reference feeds positions = len(seq) in decode (model_runner.py:219)
+    # Decode steps of sequences that can only end by length (ignore_eos) are launched before the token ids of
+    # the step before them have been read back: the ids stay on the device as the next step's input, the host
+    # keeps two steps in flight and patches the values into its sequences as they arrive.  Same tokens, same
+    # block ids and step counts as the step-by-step loop; False restores that loop.
+    run_ahead: bool = True
 
     def __post_init__(self):
         if isinstance(self.model, str) and self.model.lower() in QWEN3_SHAPES:

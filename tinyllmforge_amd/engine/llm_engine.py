@@ -5,6 +5,7 @@ configurations are random-init models without tokenizer files)."""
 from __future__ import annotations
 
 import atexit
+from collections import deque
 from dataclasses import fields
 from time import perf_counter
 
@@ -32,6 +33,10 @@ class LLMEngine:
                 config.eos = self.tokenizer.eos_token_id
         self.scheduler = Scheduler(config)
         self.last_stats = {}
+        # decode steps whose token ids have not been read back yet, oldest first:
+        # (sequences, device ids, pinned landing buffer, arrival event, seq_id -> row)
+        self._ahead = deque()
+        self.steps_ahead = 0     # decode steps launched without waiting for the ids of the step before
         atexit.register(self.exit)
 
     def exit(self):
@@ -49,11 +54,48 @@ class LLMEngine:
                              f"({self.config.hf_config.max_position_embeddings}): no RoPE row for its tail")
         self.scheduler.add(Sequence(prompt, sampling_params))
 
+    AHEAD = 2    # decode steps in flight before the oldest one's token ids are waited for
+
+    def _retire(self):
+        """Read back the oldest step that ran ahead; the sequences it finished, now that their ids are known."""
+        seqs, _, landing, arrived, _ = self._ahead.popleft()
+        arrived.synchronize()
+        self.scheduler.patch(seqs, landing.tolist())
+        return [(s.seq_id, s.completion_token_ids) for s in seqs if s.is_finished and s.num_unknown == 0]
+
+    def _drain(self):
+        outputs = []
+        while self._ahead:
+            outputs += self._retire()
+        return outputs
+
     def step(self):
-        seqs, is_prefill = self.scheduler.schedule()
-        token_ids = self.model_runner.call("run", seqs, is_prefill)
-        self.scheduler.postprocess(seqs, token_ids)
-        outputs = [(s.seq_id, s.completion_token_ids) for s in seqs if s.is_finished]
+        """One engine step (llm_engine.py:53-59).  A decode step of sequences that can only end by length
+        does not wait for its token ids (Config.run_ahead): it is launched with the ids of the step before it
+        still on the device, and the sequences finished by a step are reported when its ids have arrived -
+        at the latest by the step that finishes the last sequence."""
+        runner, sched = self.model_runner, self.scheduler
+        ahead = self.config.run_ahead and sched.can_run_ahead() and bool(runner.graph_bs) and not runner.enforce_eager
+        outputs = [] if ahead else self._drain()
+        seqs, is_prefill = sched.schedule()
+        if ahead and not is_prefill and runner.graph_ready(seqs):
+            while len(self._ahead) >= self.AHEAD:
+                outputs += self._retire()
+            feed = None
+            if self._ahead:      # the ids this step feeds on are those of the newest step in flight
+                _, tokens, _, _, rows = self._ahead[-1]
+                feed = (tokens, [rows[s.seq_id] for s in seqs])
+            tokens, landing, arrived = runner.run_ahead(seqs, feed)
+            self._ahead.append((seqs, tokens, landing, arrived, {s.seq_id: i for i, s in enumerate(seqs)}))
+            sched.postprocess_ahead(seqs)
+            self.steps_ahead += 1
+            if sched.is_finished():
+                outputs += self._drain()
+        else:
+            outputs += self._drain()
+            token_ids = runner.call("run", seqs, is_prefill)
+            sched.postprocess(seqs, token_ids)
+            outputs += [(s.seq_id, s.completion_token_ids) for s in seqs if s.is_finished]
         num_tokens = sum(len(s) for s in seqs) if is_prefill else -len(seqs)
         # for the statistics of generate(): cached prompt tokens of a prefill step, context tokens a
         # decode step's attention reads (the token stored in this step included)
@@ -62,7 +104,7 @@ class LLMEngine:
         return outputs, num_tokens
 
     def is_finished(self):
-        return self.scheduler.is_finished()
+        return self.scheduler.is_finished() and not self._ahead
 
     def generate(self, prompts, sampling_params, use_tqdm: bool = False):
         if not isinstance(sampling_params, list):

@@ -70,7 +70,7 @@ class ModelRunner:
         """Release the graphs, the KV pool and the weights (whoever still holds this object holds no memory)."""
         torch.cuda.synchronize()
         self.graphs.clear()
-        self.graph_vars = self.graph_host = self.graph_pack_dev = self.graph_pack_host = None
+        self.graph_vars = self.graph_ring = self.graph_pack_dev = None
         if getattr(self, "model", None) is not None:
             for module in self.model.modules():
                 if hasattr(module, "k_cache") and hasattr(module, "v_cache"):
@@ -250,22 +250,37 @@ class ModelRunner:
     def run_model(self, input_ids, positions, is_prefill):
         return self.model.compute_logits(self.run_hidden(input_ids, positions, is_prefill))
 
+    RING = 4   # pinned mirrors of the graphs' static inputs (two steps in flight + the one being filled + slack)
+
+    def graph_ready(self, seqs) -> bool:
+        """Whether a decode step over ``seqs`` fits the captured graphs (batch bucket, block-table width)."""
+        return bool(not self.enforce_eager and self.graph_bs and len(seqs) <= self.graph_bs[-1]
+                    and max(len(s.block_table) for s in seqs) <= self.graph_max_blocks)
+
     @torch.inference_mode()
-    def run_decode_graph(self, seqs):
+    def launch_decode_graph(self, seqs, feed=None):
         """Decode step through a captured graph: the integer inputs (I.decode_inputs, the same function the
-        eager path uploads) are written straight into the pinned mirror of the graph's static buffers,
+        eager path uploads) are written straight into a pinned mirror of the graph's static buffers,
         padding rows get slot -1 (no cache write) and length 0 (no cache read), one H2D copy, replay.
-        Returns the final hidden states."""
+        ``feed = (token ids of the step before on the device, row of each of this step's sequences in that
+        step)`` takes the input ids from there instead of from the host (whose sequences do not know them
+        yet).  Returns the final hidden states (the graphs' static output buffer)."""
         bs = len(seqs)
         gbs = next(x for x in self.graph_bs if x >= bs)
         d = I.decode_inputs(seqs, self.block_size, self.config.decode_position_quirk)
-        h = self.graph_host
+        slot = self.graph_ring[self.graph_ring_at]
+        self.graph_ring_at = (self.graph_ring_at + 1) % self.RING
+        if slot["copied"] is not None:
+            slot["copied"].synchronize()      # the copy out of this mirror, four steps ago, has long run
+        h = slot["views"]
         h["input_ids"][:bs] = d["input_ids"]
         h["positions"][:bs] = d["positions"]
         h["slot_mapping"][:bs] = d["slot_mapping"]
         h["context_lens"][:bs] = d["context_lens"]
         w = d["block_tables"].shape[1]
         h["block_tables"][:bs, :w] = d["block_tables"]
+        if feed is not None:
+            h["feed_index"][:bs] = feed[1]
         if gbs != bs:
             h["input_ids"][bs:gbs] = 0
             h["positions"][bs:gbs] = 0
@@ -276,10 +291,34 @@ class ModelRunner:
         if t is not None:
             h["temperatures"][:bs] = t
             self._temperatures = self.graph_vars["temperatures"][:bs]
-        self.graph_pack_dev.copy_(self.graph_pack_host, non_blocking=True)
+        self.graph_pack_dev.copy_(slot["pack"], non_blocking=True)
+        if slot["copied"] is None:
+            slot["copied"] = torch.cuda.Event()
+        slot["copied"].record()
+        if feed is not None:
+            torch.index_select(feed[0], 0, self.graph_vars["feed_index"][:bs], out=self.graph_vars["input_ids"][:bs])
         set_context(False)
         self.graphs[gbs].replay()
-        return self.graph_vars["outputs"][:bs]
+        return self.graph_vars["outputs"][:bs], slot
+
+    def run_decode_graph(self, seqs):
+        return self.launch_decode_graph(seqs)[0]
+
+    @torch.inference_mode()
+    def run_ahead(self, seqs, feed=None):
+        """One graph decode step whose token ids stay on the device: returns them with the pinned buffer their
+        copy lands in and the event that says when.  Nothing here waits for the GPU."""
+        hidden, slot = self.launch_decode_graph(seqs, feed)
+        if self._all_greedy and self.fused_greedy:
+            tokens = self.model.compute_greedy_ids(hidden)
+        else:
+            tokens = self.sampler(self.model.compute_logits(hidden), self._temperatures, self._all_greedy)
+        reset_context()
+        landing = slot["tokens"][:len(seqs)]
+        landing.copy_(tokens, non_blocking=True)
+        arrived = torch.cuda.Event()
+        arrived.record()
+        return tokens, landing, arrived
 
     @torch.inference_mode()
     def sample(self, hidden, temperatures):
@@ -291,9 +330,7 @@ class ModelRunner:
         return self.sampler(self.model.compute_logits(hidden), temperatures, self._all_greedy).tolist()
 
     def run(self, seqs, is_prefill):
-        use_graph = (not is_prefill and not self.enforce_eager and self.graph_bs
-                     and len(seqs) <= self.graph_bs[-1]
-                     and max(len(s.block_table) for s in seqs) <= self.graph_max_blocks)
+        use_graph = not is_prefill and self.graph_ready(seqs)
         if use_graph:
             hidden = self.run_decode_graph(seqs)
             token_ids = self.sample(hidden, self.prepare_sample(seqs))
@@ -321,6 +358,7 @@ class ModelRunner:
         # device-side copies or fills between the replays.
         layout, off = {}, 0
         for name, dt, shape in (("input_ids", torch.int64, (max_bs,)), ("positions", torch.int64, (max_bs,)),
+                                ("feed_index", torch.int64, (max_bs,)),
                                 ("slot_mapping", torch.int32, (max_bs,)), ("context_lens", torch.int32, (max_bs,)),
                                 ("temperatures", torch.float32, (max_bs,)),
                                 ("block_tables", torch.int32, (max_bs, max_blocks))):
@@ -328,15 +366,23 @@ class ModelRunner:
             layout[name] = (off, nbytes, dt, shape)
             off += (nbytes + 15) // 16 * 16
         self.graph_pack_dev = torch.zeros(off, dtype=torch.uint8, device=dev)
-        self.graph_pack_host = torch.zeros(off, dtype=torch.uint8, pin_memory=True)
-        host_np = self.graph_pack_host.numpy()
+        # A ring of pinned mirrors: a step that runs ahead fills the next mirror while the copy out of the
+        # previous one may still be queued behind the graph before it; an event per mirror says when its
+        # copy has run.  The token ids of a step come back through a ring of pinned buffers of their own.
         np_dt = {torch.int64: np.int64, torch.int32: np.int32, torch.float32: np.float32}
-        gv, self.graph_host = {}, {}
+        self.graph_ring = []
+        for _ in range(self.RING):
+            pack = torch.zeros(off, dtype=torch.uint8, pin_memory=True)
+            host_np = pack.numpy()
+            views = {name: host_np[o:o + nbytes].view(np_dt[dt]).reshape(shape) for name, (o, nbytes, dt, shape) in layout.items()}
+            views["slot_mapping"][:] = -1
+            self.graph_ring.append(dict(pack=pack, views=views, copied=None,
+                                        tokens=torch.zeros(max_bs, dtype=torch.int64, pin_memory=True)))
+        self.graph_ring_at = 0
+        gv = {}
         for name, (o, nbytes, dt, shape) in layout.items():
             gv[name] = self.graph_pack_dev[o:o + nbytes].view(dt).view(*shape)
-            self.graph_host[name] = host_np[o:o + nbytes].view(np_dt[dt]).reshape(shape)
-        self.graph_host["slot_mapping"][:] = -1
-        self.graph_pack_dev.copy_(self.graph_pack_host)
+        self.graph_pack_dev.copy_(self.graph_ring[0]["pack"])
         gv["outputs"] = torch.zeros(max_bs, hf.hidden_size, dtype=hf.torch_dtype, device=dev)
         self.graph_max_blocks = max_blocks
         self.graph_bs = [b for b in (1, 2, 4, 8) if b <= max_bs] + list(range(16, max_bs + 1, 16))

@@ -83,3 +83,33 @@ class Scheduler:
                 seq.status = SequenceStatus.FINISHED
                 self.block_manager.deallocate(seq)
                 self.running.remove(seq)
+
+    # -- a decode step that runs ahead of the read-back of its tokens (no counterpart in the reference, whose
+    #    step waits for its token ids): legal while no sequence of the step can end on a token VALUE
+    def can_run_ahead(self) -> bool:
+        """The next step is a decode step (nothing waits, or the head of the queue does not fit now: the same test
+        as in ``_admit_waiting``) of sequences that ignore EOS."""
+        if not self.running or not all(s.ignore_eos for s in self.running):
+            return False
+        if self.waiting and self.max_num_seqs > 0:
+            head = self.waiting[0]
+            if len(head) <= self.max_num_batched_tokens and self.block_manager.can_allocate(head):
+                return False
+        return True
+
+    def postprocess_ahead(self, seqs: list[Sequence]):
+        """``postprocess`` without the token values: lengths, finishing by length and block release as there;
+        the values follow through ``patch``."""
+        for seq in seqs:
+            assert seq.ignore_eos
+            seq.append_unknown()
+            if seq.num_completion_tokens == seq.max_tokens or len(seq) >= self.max_len:
+                seq.status = SequenceStatus.FINISHED
+                self.block_manager.deallocate(seq)
+                self.running.remove(seq)
+
+    def patch(self, seqs: list[Sequence], token_ids: list[int]):
+        """The token values of the oldest step that ran ahead, then the seals that waited for them."""
+        for seq, tok in zip(seqs, token_ids):
+            seq.patch_oldest_unknown(tok)
+        self.block_manager.seal_known()

@@ -30,6 +30,9 @@ class Sequence:
         self.num_tokens = self.num_prompt_tokens
         self.last_token = self.token_ids[-1]
         self.num_cached_tokens = 0
+        # tokens at the tail whose values are not on the host yet (a decode step that runs ahead of the
+        # read-back of the step before it appends a stand-in and patches the value in later)
+        self.num_unknown = 0
         self.block_table: list[int] = []
         self.temperature = sp.temperature
         self.max_tokens = sp.max_tokens
@@ -77,3 +80,22 @@ class Sequence:
         self.token_ids.append(token_id)
         self.last_token = token_id
         self.num_tokens += 1
+
+    def append_unknown(self):
+        """Lengthen the sequence by a token whose value arrives later (``patch_oldest_unknown``)."""
+        self.token_ids.append(0)
+        self.last_token = 0
+        self.num_tokens += 1
+        self.num_unknown += 1
+
+    def patch_oldest_unknown(self, token_id: int):
+        assert self.num_unknown > 0
+        at = self.num_tokens - self.num_unknown
+        self.token_ids[at] = token_id
+        if at == self.num_tokens - 1:
+            self.last_token = token_id
+        self.num_unknown -= 1
+
+    @property
+    def num_known_tokens(self):
+        return self.num_tokens - self.num_unknown
