@@ -563,12 +563,15 @@ def bench_e2e(args, quantization):
     sps = [SamplingParams(temperature=0.0, ignore_eos=True, max_tokens=m) for m in max_tokens]
     for _ in range(max(1, args.warmup)):
         llm.generate([[1, 2, 3, 4, 5, 6, 7, 8]], SamplingParams(temperature=0.0, max_tokens=8, ignore_eos=True))
+    ahead0 = llm.steps_ahead
     st, wall, at_mark = timed_generate(llm, prompts, sps, args.steps)
+    steps_ahead = llm.steps_ahead - ahead0
     total = sum(max_tokens)                  # every sequence runs to its max_tokens (ignore_eos)
     all_steps = st["prefill_steps"] + st["decode_steps"]
     stats = dict(steps=all_steps, prefill_steps=st["prefill_steps"], decode_steps=st["decode_steps"],
                  prefill_s=round(st["prefill_time"], 3), decode_s=round(st["decode_time"], 3),
                  decode_ms_per_step=round(1e3 * st["decode_time"] / max(1, st["decode_steps"]), 3),
+                 decode_steps_run_ahead=steps_ahead,     # launched before the ids of the step before were read back
                  decode_byte_floor=decode_byte_floor(llm.config.hf_config, st, quantization, kv_itemsize=2))
     if args.steps > 0 and at_mark is not None:
         slice_steps, slice_s = args.steps, at_mark

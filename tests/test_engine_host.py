@@ -321,3 +321,93 @@ def test_safetensors_loader_and_offline_int8_checkpoint(tmp_path):
         assert la.mlp.gate_up_proj.interleaved and lb.mlp.gate_up_proj.interleaved
     assert torch.equal(a.model.embed_tokens.weight, b.model.embed_tokens.weight)
     assert torch.equal(a.lm_head.weight, b.lm_head.weight) and torch.equal(a.model.norm.weight, b.model.norm.weight)
+
+
+# ----------------------------------------------------------------------------- decode steps that run ahead
+def _simulate(ahead, depth, nblk, seed, block_size=16):
+    """The engine loop without a model: a step's tokens are a fixed function of (sequence, length), and in the
+    run-ahead form they reach the scheduler ``depth`` steps late (postprocess_ahead now, patch later)."""
+    import itertools
+    import random
+    from collections import deque
+    from tinyllmforge_amd.config import Config
+    from tinyllmforge_amd.engine.block_manager import BlockManager
+    from tinyllmforge_amd.engine.scheduler import Scheduler
+    from tinyllmforge_amd.engine.sequence import Sequence
+    from tinyllmforge_amd.sampling_params import SamplingParams
+    rnd = random.Random(seed)
+    cfg = Config("qwen3-0.6b", num_kvcache_blocks=nblk, max_num_seqs=8, max_num_batched_tokens=4096, max_model_len=2048)
+    old_bs, old_ids = Sequence.block_size, Sequence._ids
+    Sequence.block_size, Sequence._ids = block_size, itertools.count(1000)
+    try:
+        sch = Scheduler(cfg)
+        sch.block_manager = BlockManager(nblk, block_size)
+        seqs = [Sequence([rnd.randint(0, 99) for _ in range(rnd.randint(3, 60))],
+                         SamplingParams(temperature=0.0, max_tokens=rnd.randint(5, 90), ignore_eos=True)) for _ in range(12)]
+        for s in seqs:
+            sch.add(s)
+        tok = lambda s, n: (s.seq_id * 7919 + n * 31) % 1000
+        inflight, trace, ran_ahead = deque(), [], 0
+        while not sch.is_finished() or inflight:
+            if sch.is_finished():
+                sch.patch(*inflight.popleft())
+                continue
+            if ahead and sch.can_run_ahead():
+                while len(inflight) >= depth:
+                    sch.patch(*inflight.popleft())
+                batch, prefill = sch.schedule()
+                assert not prefill
+                trace.append(("d", [s.seq_id for s in batch], [list(s.block_table) for s in batch]))
+                inflight.append((batch, [tok(s, len(s)) for s in batch]))
+                sch.postprocess_ahead(batch)
+                ran_ahead += 1
+            else:
+                while inflight:
+                    sch.patch(*inflight.popleft())
+                batch, prefill = sch.schedule()
+                trace.append(("p" if prefill else "d", [s.seq_id for s in batch], [list(s.block_table) for s in batch]))
+                sch.postprocess(batch, [tok(s, len(s)) for s in batch])
+        bm = sch.block_manager
+        assert not bm.unsealed and not bm.used_block_ids and all(s.num_unknown == 0 for s in seqs)
+        return dict(trace=trace, tokens=[s.token_ids for s in seqs], hashes=dict(bm.hash_to_block_id),
+                    free=list(bm.free_block_ids), blocks=[(b.hash, b.token_ids) for b in bm.blocks], ran_ahead=ran_ahead)
+    finally:
+        Sequence.block_size, Sequence._ids = old_bs, old_ids
+
+
+@pytest.mark.parametrize("nblk", [40, 14, 9])
+@pytest.mark.parametrize("depth", [1, 2, 4])
+def test_run_ahead_bookkeeping_equals_the_step_by_step_loop(nblk, depth):
+    """Token values that arrive ``depth`` steps late (stand-ins appended, values patched in, full blocks sealed when
+    their tokens are known) leave every step's sequences and block tables, the token lists, the prefix-cache hashes,
+    the free list and the blocks exactly as the step-by-step loop does: with room to spare (40 blocks of 16 tokens),
+    with preemption (14) and with most sequences waiting most of the time (9)."""
+    for seed in range(4):
+        a = _simulate(False, depth, nblk, seed)
+        b = _simulate(True, depth, nblk, seed)
+        for key in ("trace", "tokens", "hashes", "free", "blocks"):
+            assert a[key] == b[key], (key, seed)
+        decode_steps = sum(1 for t in a["trace"] if t[0] == "d")
+        assert a["ran_ahead"] == 0 and b["ran_ahead"] == decode_steps > 50
+    if nblk < 40:
+        assert sum(1 for t in a["trace"] if t[0] == "p") > 3      # preempted sequences were prefilled again
+
+
+def test_run_ahead_is_refused_when_a_sequence_may_end_on_a_token_value():
+    from tinyllmforge_amd.config import Config
+    from tinyllmforge_amd.engine.scheduler import Scheduler
+    from tinyllmforge_amd.engine.sequence import Sequence
+    from tinyllmforge_amd.sampling_params import SamplingParams
+    sch = Scheduler(Config("qwen3-0.6b", num_kvcache_blocks=8, max_num_seqs=4, max_model_len=1024))
+    a = Sequence([1, 2, 3], SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True))
+    b = Sequence([4, 5, 6], SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=False))
+    sch.add(a)
+    assert not sch.can_run_ahead()                 # a prefill comes first
+    batch, prefill = sch.schedule()
+    sch.postprocess(batch, [7])
+    assert prefill and sch.can_run_ahead()
+    sch.add(b)
+    assert not sch.can_run_ahead()                 # the newcomer fits: the next step is its prefill
+    batch, prefill = sch.schedule()
+    sch.postprocess(batch, [8])
+    assert prefill and not sch.can_run_ahead()     # b may end on EOS
