@@ -324,9 +324,11 @@ def test_safetensors_loader_and_offline_int8_checkpoint(tmp_path):
 
 
 # ----------------------------------------------------------------------------- decode steps that run ahead
-def _simulate(ahead, depth, nblk, seed, block_size=16):
+def _simulate(ahead, depth, nblk, seed, block_size=16, arrivals=False):
     """The engine loop without a model: a step's tokens are a fixed function of (sequence, length), and in the
-    run-ahead form they reach the scheduler ``depth`` steps late (postprocess_ahead now, patch later)."""
+    run-ahead form they reach the scheduler ``depth`` steps late (postprocess_ahead now, patch later).
+    ``arrivals``: five of the twelve requests are added while the loop runs (after a given number of steps, or when
+    the engine falls idle), two of them may end on EOS, and one of those does."""
     import itertools
     import random
     from collections import deque
@@ -344,12 +346,25 @@ def _simulate(ahead, depth, nblk, seed, block_size=16):
         sch.block_manager = BlockManager(nblk, block_size)
         seqs = [Sequence([rnd.randint(0, 99) for _ in range(rnd.randint(3, 60))],
                          SamplingParams(temperature=0.0, max_tokens=rnd.randint(5, 90), ignore_eos=True)) for _ in range(12)]
-        for s in seqs:
-            sch.add(s)
         tok = lambda s, n: (s.seq_id * 7919 + n * 31) % 1000
+        pending = []
+        if arrivals:
+            for s in (seqs[8], seqs[10]):
+                s.ignore_eos = False
+            sch.eos = tok(seqs[8], len(seqs[8]) + 4)      # the fifth token of seqs[8]
+            pending = list(zip((10, 25, 25, 60, 100), seqs[7:]))
+            seqs_at_start = seqs[:7]
+        else:
+            seqs_at_start = seqs
+        for s in seqs_at_start:
+            sch.add(s)
         inflight, trace, ran_ahead = deque(), [], 0
-        while not sch.is_finished() or inflight:
+        while True:
+            while pending and (pending[0][0] <= len(trace) or sch.is_finished()):
+                sch.add(pending.pop(0)[1])
             if sch.is_finished():
+                if not inflight:
+                    break
                 sch.patch(*inflight.popleft())
                 continue
             if ahead and sch.can_run_ahead():
@@ -370,7 +385,8 @@ def _simulate(ahead, depth, nblk, seed, block_size=16):
         bm = sch.block_manager
         assert not bm.unsealed and not bm.used_block_ids and all(s.num_unknown == 0 for s in seqs)
         return dict(trace=trace, tokens=[s.token_ids for s in seqs], hashes=dict(bm.hash_to_block_id),
-                    free=list(bm.free_block_ids), blocks=[(b.hash, b.token_ids) for b in bm.blocks], ran_ahead=ran_ahead)
+                    free=list(bm.free_block_ids), blocks=[(b.hash, b.token_ids) for b in bm.blocks], ran_ahead=ran_ahead,
+                    ended_on_eos=[s.seq_id for s in seqs if not s.ignore_eos and s.num_completion_tokens < s.max_tokens])
     finally:
         Sequence.block_size, Sequence._ids = old_bs, old_ids
 
@@ -391,6 +407,21 @@ def test_run_ahead_bookkeeping_equals_the_step_by_step_loop(nblk, depth):
         assert a["ran_ahead"] == 0 and b["ran_ahead"] == decode_steps > 50
     if nblk < 40:
         assert sum(1 for t in a["trace"] if t[0] == "p") > 3      # preempted sequences were prefilled again
+
+
+@pytest.mark.parametrize("nblk", [40, 12])
+def test_run_ahead_with_requests_that_arrive_while_steps_are_in_flight(nblk):
+    """Requests added between steps (a serving loop) while decode steps are in flight: the loop drains and takes the
+    newcomer's prefill exactly where the step-by-step loop does; while a sequence that may end on EOS is running no
+    step runs ahead, and after it has ended (one does end on EOS, at its fifth token) the steps run ahead again."""
+    for seed in range(4):
+        a = _simulate(False, 2, nblk, seed, arrivals=True)
+        b = _simulate(True, 2, nblk, seed, arrivals=True)
+        for key in ("trace", "tokens", "hashes", "free", "blocks"):
+            assert a[key] == b[key], (key, seed)
+        decode_steps = sum(1 for t in a["trace"] if t[0] == "d")
+        assert a["ran_ahead"] == 0 and 10 < b["ran_ahead"] < decode_steps
+        assert len(a["ended_on_eos"]) >= 1 and a["ended_on_eos"] == b["ended_on_eos"]
 
 
 def test_run_ahead_is_refused_when_a_sequence_may_end_on_a_token_value():
