@@ -53,7 +53,7 @@ def parse():
                     help="engine steps that steps/ms_per_step describe (0 = all); value is always the whole job")
     ap.add_argument("--warmup", type=int, default=1, help="warm-up generate() calls before the timed run")
     ap.add_argument("--workload", default="e2e",
-                    choices=["e2e", "decode_attn", "gemm", "prefill_attn", "elementwise", "c5", "all"])
+                    choices=["e2e", "decode_attn", "gemm", "prefill_attn", "elementwise", "clock", "c5", "all"])
     ap.add_argument("--attn-steps", type=int, default=200, help="timed launches of the decode-attention microbench")
     ap.add_argument("--num-seqs", type=int, default=256)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -193,6 +193,93 @@ def bench_probes(args):
                                       note="4 waves per CU stream from HBM, 4 re-read 1 MiB out of L2; loads return in "
                                            "order through a CU's L1, so the two do not overlap")
     return res
+
+
+def bench_clock(args, seconds=2.0):
+    """The shader clock the part holds under each load, read from ``rocm-smi --showclocks`` (a child process polled
+    from a thread) while the load runs back to back: the register-only MFMA stream on small integers and on random
+    operands, the W8A16 GEMM of the gate_up projection at 8192 tokens on random and on small-integer data, and the
+    paged decode attention microbench.  The matrix-core peak scales with that clock (2.5 PFLOP/s is at 2.4 GHz)."""
+    import re
+    import shutil
+    import subprocess
+    import threading
+    import torch
+    from tinyllmforge_amd import _lib, ops as P
+    smi = shutil.which("rocm-smi") or "/opt/rocm/bin/rocm-smi"
+    if not os.path.exists(smi):
+        return {"skipped": "rocm-smi not found"}
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+
+    def read_sclk():
+        try:
+            r = subprocess.run([smi, "--showclocks"], capture_output=True, text=True, timeout=10)
+        except Exception:
+            return None
+        for line in r.stdout.splitlines():
+            if "sclk" in line:
+                m = re.search(r"\((\d+)Mhz\)", line)
+                if m:
+                    return int(m.group(1))
+        return None
+
+    def under_load(fn, work_per_call):
+        stop, seen = threading.Event(), []
+
+        def poll():
+            while not stop.is_set():
+                v = read_sclk()
+                if v is not None:
+                    seen.append(v)
+        fn()
+        torch.cuda.synchronize()
+        th = threading.Thread(target=poll)
+        th.start()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0, calls, gpu_ms = time.perf_counter(), 0, 0.0
+        while time.perf_counter() - t0 < seconds:
+            a.record()
+            for _ in range(10):
+                fn()
+            b.record()
+            torch.cuda.synchronize()
+            gpu_ms += a.elapsed_time(b)
+            calls += 10
+        stop.set()
+        th.join()
+        body = seen[1:] or seen            # the first reading may predate the load
+        mhz = sorted(body)[len(body) // 2] if body else None
+        return mhz, work_per_call * calls / (gpu_ms * 1e-3)
+
+    out = {"idle_sclk_MHz": read_sclk(), "loads": []}
+    buf = torch.empty(512 * 256, dtype=torch.float32, device="cuda")
+    iters = 4000
+    flop = 2.0 * 32 * 32 * 16 * 16 * iters * 2048
+    for mode, name in ((0, "mfma stream, small integers"), (1, "mfma stream, random operands"),
+                       (3, "mfma stream, random operands, idle cycles after every MFMA")):
+        mhz, rate = under_load(lambda: _lib.check(lib.tlf_probe_mfma(buf.data_ptr(), iters, mode, st), "probe"), flop)
+        out["loads"].append(dict(load=name, sclk_MHz=mhz, TFLOPs=round(rate / 1e12, 1)))
+    N, K, M = 24576, 4096, 8192
+    g = torch.Generator(device="cuda").manual_seed(0)
+    sc = torch.rand(N, device="cuda", generator=g) * 0.01
+    for name, lo, hi, xs in (("W8A16 GEMM gate_up 8192 tokens, random data", -127, 128, None),
+                             ("W8A16 GEMM gate_up 8192 tokens, small integers", -2, 3, 2)):
+        w = P.pack_w8(torch.randint(lo, hi, (N, K), dtype=torch.int8, device="cuda", generator=g))
+        x = (torch.randn(M, K, device="cuda", generator=g) if xs is None else
+             torch.randint(-xs, xs + 1, (M, K), device="cuda", generator=g).float()).to(torch.bfloat16)
+        mhz, rate = under_load(lambda: P.w8a16_linear(x, w, sc), 2.0 * M * N * K)
+        out["loads"].append(dict(load=name, sclk_MHz=mhz, TFLOPs=round(rate / 1e12, 1)))
+        del w, x
+    case = make_decode_case(batch=args.batch)
+    mhz, rate = under_load(lambda: P.paged_decode_attention(case["q"], case["k_cache"], case["v_cache"], case["ctx"], case["bt"],
+                                                            case["scale"], **case["scales"]), case["algo_bytes"])
+    out["loads"].append(dict(load="paged decode attention, configs[1]", sclk_MHz=mhz, GBps=round(rate / 1e9, 1)))
+    for r in out["loads"]:
+        if r.get("TFLOPs") and r["sclk_MHz"]:
+            # share of what the matrix cores could do at the clock the part held
+            r["of_peak_at_that_clock"] = round(r["TFLOPs"] / (MFMA_BF16_PEAK_TFLOPS * r["sclk_MHz"] / 2400.0), 3)
+    return out
 
 
 def bench_decode_attn(args, fp8=False, hq=32):
@@ -674,6 +761,17 @@ def main():
             "roofline": roofline, "cpu_baseline": None if args.no_cpu_baseline else cpu_baseline_gemm(),
             "extra": extra}))
         return
+    if args.workload == "clock":   # its own line: the shader clock under each load
+        clk = bench_clock(args)
+        extra["clock_probe"] = clk
+        gemm = next((r for r in clk.get("loads", []) if "random data" in r["load"]), None)
+        print(json.dumps({
+            "metric": "W8A16 GEMM TFLOP/s vs bf16 MFMA peak", "value": gemm and gemm["TFLOPs"], "unit": "TFLOP/s", "n_gpus": 1,
+            "steps": None, "warmup": 1, "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16", "data": "synthetic",
+            "config": {"workload": "shader clock (rocm-smi) under the MFMA stream, the gate_up GEMM at 8192 tokens and decode attention"},
+            "roofline": roofline, "cpu_baseline": None, "extra": extra}))
+        return
     if args.workload == "elementwise":   # its own line: the single-pass kernels
         rows = bench_elementwise(args)
         extra["elementwise"] = rows
@@ -719,6 +817,7 @@ def main():
     if args.workload == "e2e" and not args.skip_gemm:
         extra["w8a16_gemm"] = bench_gemm(args)          # BASELINE.json configs[2]
         extra["elementwise"] = bench_elementwise(args)
+        extra["clock_probe"] = bench_clock(args)
     # the decode microbench on e4m3 rows with 64 query heads (the 32B shape's attention)
     a8 = bench_decode_attn(args, fp8=True, hq=64)
     a8.pop("case")

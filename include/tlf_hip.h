@@ -427,7 +427,8 @@ int tlf_probe_copy(const void *src, void *dst, size_t bytes, void *stream);
 /* Two more probes for the GEMM's rooflines (no reference counterpart).
  * tlf_probe_mfma: 512 workgroups x 4 waves each issue 16 * iters v_mfma_f32_32x32x16_bf16 from registers:
  *   2 * 32*32*16 * 16 * iters * 2048 flop per launch.  mode 0: small-integer operands, mode 1: pseudo-random
- *   bf16 values times int8-valued weights (the clock a kernel sees on real data).  out: 512 * 256 floats.
+ *   bf16 values times int8-valued weights (the clock a kernel sees on real data); mode 2 / 3: the same two with
+ *   idle cycles after every MFMA (a duty of about 0.9: how the clock answers to the load).  out: 512 * 256 floats.
  * tlf_probe_mix: 256 workgroups of 8 waves; waves 0..3 stream big (read once: floor(big_bytes / 16 MiB) * 16 KiB
  *   per wave, from HBM), waves 4..7 re-read small_region (L2 resident: at least 16 KiB, a multiple of 1 KiB)
  *   l2_eighths / 8 times as many bytes.  Shows what a CU's vector-memory path does with both at once. */

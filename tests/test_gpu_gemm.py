@@ -372,3 +372,22 @@ def test_lm_head_with_greedy_sample_equals_gemm_then_argmax(M, N, K):
     top = ref.max(-1).values
     got = ref.gather(1, which[ids][:, None])[:, 0]
     assert ((top - got) <= O.bf16_ulp(top)).all()                      # and that group is the oracle's maximum
+
+
+def test_mfma_probe_modes_compute_the_same_sums():
+    """The register-only MFMA stream behind the GEMM's roofline: with idle cycles after every MFMA (modes 2, 3) the
+    accumulators end with the same values as without (modes 0, 1): on small integers the sums are exact, on the
+    pseudo-random operands the same instructions run in the same order.  Mode 0 in closed form for one lane: every
+    MFMA adds sum_k a[k] b[k] over 16 k to each accumulator entry, 16 * iters times, 64 entries per lane."""
+    from tinyllmforge_amd import _lib
+    lib = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    outs = []
+    for mode in range(4):
+        out = torch.full((512 * 256,), float("nan"), dtype=torch.float32, device=DEV)
+        _lib.check(lib.tlf_probe_mfma(out.data_ptr(), 3, mode, st), "probe")
+        outs.append(out.cpu())
+    assert torch.equal(outs[0], outs[2]) and torch.equal(outs[1], outs[3])
+    assert torch.isfinite(outs[1]).all() and not torch.equal(outs[0], outs[1])
+    assert (outs[0] == outs[0].round()).all() and outs[0].min() >= 0 and outs[0].max() > 0
+    assert lib.tlf_probe_mfma(out.data_ptr(), 3, 4, st) != 0          # no such mode

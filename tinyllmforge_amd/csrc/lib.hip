@@ -73,17 +73,19 @@ __global__ __launch_bounds__(256) void probe_copy_kernel(const uint4 *__restrict
 
 // Register-only MFMA stream: what the matrix cores sustain with nothing to wait for.  Every wave issues
 // 16 * iters v_mfma_f32_32x32x16_bf16 on four independent accumulators from operands that never change:
-// small integers (mode 0) or pseudo-random bf16 activations times int8-valued weights (mode 1).  The two
-// differ on this part: the clock drops under the switching activity of random data.
+// small integers (mode 0, 2) or pseudo-random bf16 activations times int8-valued weights (mode 1, 3).  The two
+// differ on this part: the clock drops under the switching activity of random data.  Modes 2 and 3 leave idle
+// cycles after every MFMA.
 __global__ __launch_bounds__(256) void probe_mfma_kernel(float *__restrict__ out, int iters, int mode) {
   bf16x8 a, b;
   unsigned int h = threadIdx.x * 2654435761u + blockIdx.x * 40503u + 17u;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     h = h * 1664525u + 1013904223u;
-    const float fa = mode ? (static_cast<int>(h >> 8) % 2001 - 1000) * 1e-3f : static_cast<float>((threadIdx.x + i) & 3);
+    const bool random = mode & 1;
+    const float fa = random ? (static_cast<int>(h >> 8) % 2001 - 1000) * 1e-3f : static_cast<float>((threadIdx.x + i) & 3);
     h = h * 1664525u + 1013904223u;
-    const float fb = mode ? static_cast<float>(static_cast<int>(h >> 8) % 255 - 127) : static_cast<float>(i & 1);
+    const float fb = random ? static_cast<float>(static_cast<int>(h >> 8) % 255 - 127) : static_cast<float>(i & 1);
     a[i] = static_cast<__bf16>(fa);
     b[i] = static_cast<__bf16>(fb);
   }
@@ -92,11 +94,24 @@ __global__ __launch_bounds__(256) void probe_mfma_kernel(float *__restrict__ out
   for (int j = 0; j < 4; ++j)
 #pragma unroll
     for (int v = 0; v < 16; ++v) acc[j][v] = 0.f;
-  for (int it = 0; it < iters; ++it) {
+  if (mode & 2) {
+    // the same stream with two s_nop 7 after every MFMA: the matrix pipe runs at a duty of about 0.9, so the clock
+    // the part answers with separates the power that goes with the clock from the power that goes with the MFMAs
+#define TLF_GAPPED(J) "v_mfma_f32_32x32x16_bf16 %" #J ", %4, %5, %" #J "\n\ts_nop 7\n\ts_nop 7\n\t"
+#define TLF_GAPPED4 TLF_GAPPED(0) TLF_GAPPED(1) TLF_GAPPED(2) TLF_GAPPED(3)
+    for (int it = 0; it < iters; ++it)
+      asm volatile(TLF_GAPPED4 TLF_GAPPED4 TLF_GAPPED4 TLF_GAPPED4
+                   : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3])
+                   : "v"(a), "v"(b));
+#undef TLF_GAPPED4
+#undef TLF_GAPPED
+  } else {
+    for (int it = 0; it < iters; ++it) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < 4; ++u)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[j], 0, 0, 0);
+        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[j], 0, 0, 0);
+    }
   }
   float s = 0.f;
 #pragma unroll
@@ -146,7 +161,7 @@ __global__ __launch_bounds__(512) void probe_mix_kernel(const unsigned char *__r
 
 extern "C" int tlf_probe_mfma(void *out, int32_t iters, int32_t mode, void *stream) {
   if (!out) return TLF_E_NULL;
-  if (iters < 0 || (mode != 0 && mode != 1)) return TLF_E_SHAPE;
+  if (iters < 0 || mode < 0 || mode > 3) return TLF_E_SHAPE;
   // one workgroup of four waves per CU slot, twice the CUs: two waves per SIMD keep the pipe full
   TLF_LAUNCH(tlf::probe_mfma_kernel, dim3(512), dim3(256), 0, static_cast<hipStream_t>(stream),
                      static_cast<float *>(out), iters, mode);
