@@ -201,6 +201,8 @@ __device__ __forceinline__ void rmsnorm_finish(const float (&v)[MAXC][8], const 
       CALL(64, 1);                 \
     } else if ((cols) <= 2048) {   \
       CALL(64, 4);                 \
+    } else if ((cols) <= 4096) {   \
+      CALL(256, 2);                \
     } else if ((cols) <= 8192) {   \
       CALL(256, 4);                \
     } else {                       \

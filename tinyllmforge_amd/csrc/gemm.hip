@@ -568,6 +568,42 @@ void gemm_wstream_kernel(const GemmParams p) {
 #undef TLF_DL_AFTER_GROUP
 #undef TLF_DL_ISSUE_SETUP
 
+// s += partial_k for k = 1 .. splits - 1, in that order.  All loads go out before the first add (1, 3 or 7 at a time,
+// by a branch the whole grid takes alike): in a rolled loop each load would wait for the add before it, one memory
+// round trip per partial in kernels that last a few microseconds.  An index past the end re-reads the last partial
+// and is not added.
+template <int C, int H>
+__device__ __forceinline__ void add_partials_n(const float *src, int64_t mn, int splits, float4 (&s)[H]) {
+  float4 t[C][H];
+#pragma unroll
+  for (int u = 0; u < C; ++u)
+#pragma unroll
+    for (int h = 0; h < H; ++h) t[u][h] = *reinterpret_cast<const float4 *>(src + min(u + 1, splits - 1) * mn + 4 * h);
+#pragma unroll
+  for (int u = 0; u < C; ++u)
+    if (u + 1 < splits) {
+#pragma unroll
+      for (int h = 0; h < H; ++h) { s[h].x += t[u][h].x; s[h].y += t[u][h].y; s[h].z += t[u][h].z; s[h].w += t[u][h].w; }
+    }
+}
+// H = consecutive float4 per thread (1 or 2)
+template <int H>
+__device__ __forceinline__ void add_partials(const float *src, int64_t mn, int splits, float4 (&s)[H]) {
+  if (splits <= 2) {
+    add_partials_n<1, H>(src, mn, splits, s);
+  } else if (splits <= 4) {
+    add_partials_n<3, H>(src, mn, splits, s);
+  } else {
+    add_partials_n<7, H>(src, mn, splits, s);
+    for (int k = 8; k < splits; ++k)
+#pragma unroll
+      for (int h = 0; h < H; ++h) {
+        const float4 t = *reinterpret_cast<const float4 *>(src + k * mn + 4 * h);
+        s[h].x += t.x; s[h].y += t.y; s[h].z += t.z; s[h].w += t.w;
+      }
+  }
+}
+
 // Sum the split-K partials, apply the channel scale, round once to bf16.
 template <bool W8>
 __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmParams p) {
@@ -575,11 +611,9 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmParams p) 
   const int64_t total4 = static_cast<int64_t>(p.M) * p.N / 4;
   if (i4 >= total4) return;
   const int64_t mn = static_cast<int64_t>(p.M) * p.N;
-  float4 s = *reinterpret_cast<const float4 *>(p.partial + i4 * 4);
-  for (int k = 1; k < p.splits; ++k) {
-    const float4 t = *reinterpret_cast<const float4 *>(p.partial + k * mn + i4 * 4);
-    s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
-  }
+  float4 s1[1] = {*reinterpret_cast<const float4 *>(p.partial + i4 * 4)};
+  add_partials<1>(p.partial + i4 * 4, mn, p.splits, s1);
+  float4 s = s1[0];
   if (W8) {
     const int n = static_cast<int>((i4 * 4) % p.N);
     const float4 sc = *reinterpret_cast<const float4 *>(p.scale + n);
@@ -606,15 +640,12 @@ __global__ __launch_bounds__(256) void splitk_reduce_qknorm_rope_store_kernel(co
   const int n = head * 128 + j * 8;
   const int64_t mn = static_cast<int64_t>(p.M) * p.N;
   const float *src = p.partial + tok * p.N + n;
-  float4 s0 = *reinterpret_cast<const float4 *>(src);
-  float4 s1 = *reinterpret_cast<const float4 *>(src + 4);
-#pragma unroll 4
-  for (int k = 1; k < p.splits; ++k) {
-    const float4 t0 = *reinterpret_cast<const float4 *>(src + k * mn);
-    const float4 t1 = *reinterpret_cast<const float4 *>(src + k * mn + 4);
-    s0.x += t0.x; s0.y += t0.y; s0.z += t0.z; s0.w += t0.w;
-    s1.x += t1.x; s1.y += t1.y; s1.z += t1.z; s1.w += t1.w;
-  }
+  // the token's position and slot, then its cosines and sines, are on their way while the partials are summed
+  const QkPieceMeta meta = qk_piece_meta(tok, head, a);
+  float4 sum[2] = {*reinterpret_cast<const float4 *>(src), *reinterpret_cast<const float4 *>(src + 4)};
+  const QkPieceTable table = qk_piece_table(meta, head, j, a);
+  add_partials<2>(src, mn, p.splits, sum);
+  float4 s0 = sum[0], s1 = sum[1];
   if (W8) {
     const float4 c0 = *reinterpret_cast<const float4 *>(p.scale + n);
     const float4 c1 = *reinterpret_cast<const float4 *>(p.scale + n + 4);
@@ -623,7 +654,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_qknorm_rope_store_kernel(co
   }
   const uint4 raw = make_uint4(pack_bf16x2(s0.x, s0.y), pack_bf16x2(s0.z, s0.w), pack_bf16x2(s1.x, s1.y),
                                pack_bf16x2(s1.z, s1.w));
-  qknorm_rope_store_piece(raw, tok, head, j, a);
+  qk_piece_finish(raw, tok, head, j, meta, table, a);
 }
 
 // What follows a row-parallel projection in the decoder (o_proj, down_proj) is the residual add and
@@ -643,9 +674,11 @@ struct NormTail {
   float eps;
 };
 
-template <int TPR, int MAXC, bool W8>
-__global__ __launch_bounds__(256) void splitk_reduce_add_rmsnorm_kernel(const GemmParams p,
-                                                                        const NormTail t) {
+// C = partials loaded ahead per chunk (1, 3 or 7: splits <= 2, <= 4, more; fewer where a thread has many chunks).  Every load of the row is unconditional
+// (a chunk past the row re-reads the row's last chunk, an idle thread row 0) and stands before the first use, so all of
+// them are in flight at once; only the arithmetic and the stores are predicated.
+template <int TPR, int MAXC, bool W8, int C>
+__device__ __forceinline__ void splitk_reduce_add_rmsnorm_body(const GemmParams &p, const NormTail &t) {
   constexpr int kRowsPerBlock = 256 / TPR;
   const int tid = threadIdx.x;
   const int sub = tid % TPR;
@@ -655,27 +688,47 @@ __global__ __launch_bounds__(256) void splitk_reduce_add_rmsnorm_kernel(const Ge
   const int64_t mn = static_cast<int64_t>(p.M) * p.N;
   const int64_t off = (active ? row : 0) * p.N;
   float v[MAXC][8];
-  uint4 pw[MAXC];
+  uint4 pw[MAXC], pr[MAXC];
+  float4 ab[MAXC][2], part[MAXC][C][2], sc[MAXC][2];
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int at = min(sub + c * TPR, nchunks - 1) * 8;
+    pw[c] = *reinterpret_cast<const uint4 *>(t.weight + at);
+    pr[c] = *reinterpret_cast<const uint4 *>(t.residual + off + at);
+    const float *src = p.partial + off + at;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      ab[c][h] = *reinterpret_cast<const float4 *>(src + 4 * h);
+#pragma unroll
+      for (int u = 0; u < C; ++u)
+        part[c][u][h] = *reinterpret_cast<const float4 *>(src + min(u + 1, p.splits - 1) * mn + 4 * h);
+      if (W8) sc[c][h] = *reinterpret_cast<const float4 *>(p.scale + at + 4 * h);
+    }
+  }
   float ss = 0.f;
 #pragma unroll
   for (int c = 0; c < MAXC; ++c) {
     const int chunk = sub + c * TPR;
-    pw[c] = make_uint4(0, 0, 0, 0);
     if (active && chunk < nchunks) {
-      pw[c] = *reinterpret_cast<const uint4 *>(t.weight + chunk * 8);
-      const uint4 pr = *reinterpret_cast<const uint4 *>(t.residual + off + chunk * 8);
-      const float *src = p.partial + off + chunk * 8;
-      float4 a = *reinterpret_cast<const float4 *>(src);
-      float4 b = *reinterpret_cast<const float4 *>(src + 4);
-      for (int k = 1; k < p.splits; ++k) {
-        const float4 a2 = *reinterpret_cast<const float4 *>(src + k * mn);
-        const float4 b2 = *reinterpret_cast<const float4 *>(src + k * mn + 4);
-        a.x += a2.x; a.y += a2.y; a.z += a2.z; a.w += a2.w;
-        b.x += b2.x; b.y += b2.y; b.z += b2.z; b.w += b2.w;
+      float4 a = ab[c][0], b = ab[c][1];
+#pragma unroll
+      for (int u = 0; u < C; ++u)
+        if (u + 1 < p.splits) {
+          const float4 a2 = part[c][u][0], b2 = part[c][u][1];
+          a.x += a2.x; a.y += a2.y; a.z += a2.z; a.w += a2.w;
+          b.x += b2.x; b.y += b2.y; b.z += b2.z; b.w += b2.w;
+        }
+      {  // partials beyond those loaded ahead, one at a time
+        const float *src = p.partial + off + chunk * 8;
+        for (int k = C + 1; k < p.splits; ++k) {
+          const float4 a2 = *reinterpret_cast<const float4 *>(src + k * mn);
+          const float4 b2 = *reinterpret_cast<const float4 *>(src + k * mn + 4);
+          a.x += a2.x; a.y += a2.y; a.z += a2.z; a.w += a2.w;
+          b.x += b2.x; b.y += b2.y; b.z += b2.z; b.w += b2.w;
+        }
       }
       if (W8) {
-        const float4 s0 = *reinterpret_cast<const float4 *>(p.scale + chunk * 8);
-        const float4 s1 = *reinterpret_cast<const float4 *>(p.scale + chunk * 8 + 4);
+        const float4 s0 = sc[c][0], s1 = sc[c][1];
         a.x *= s0.x; a.y *= s0.y; a.z *= s0.z; a.w *= s0.w;
         b.x *= s1.x; b.y *= s1.y; b.z *= s1.z; b.w *= s1.w;
       }
@@ -686,7 +739,7 @@ __global__ __launch_bounds__(256) void splitk_reduce_add_rmsnorm_kernel(const Ge
       hb.w = pack_bf16x2(b.z, b.w);
       float r[8];
       unpack8(hb, v[c]);
-      unpack8(pr, r);
+      unpack8(pr[c], r);
 #pragma unroll
       for (int i = 0; i < 8; ++i) v[c][i] = __fadd_rn(v[c][i], r[i]);
       *reinterpret_cast<uint4 *>(t.residual_out + off + chunk * 8) = pack8(v[c]);
@@ -695,6 +748,18 @@ __global__ __launch_bounds__(256) void splitk_reduce_add_rmsnorm_kernel(const Ge
     }
   }
   rmsnorm_finish<TPR, MAXC>(v, pw, ss, active, sub, nchunks, p.N, t.eps, t.y + off);
+}
+
+template <int TPR, int MAXC, bool W8>
+__global__ __launch_bounds__(256) void splitk_reduce_add_rmsnorm_kernel(const GemmParams p,
+                                                                        const NormTail t) {
+  constexpr int kAhead = MAXC <= 2 ? 7 : MAXC <= 4 ? 3 : 1;   // what the registers hold: 8 x MAXC x C values per thread
+  if (p.splits <= 2 || kAhead == 1)
+    splitk_reduce_add_rmsnorm_body<TPR, MAXC, W8, 1>(p, t);
+  else if (p.splits <= 4 || kAhead == 3)
+    splitk_reduce_add_rmsnorm_body<TPR, MAXC, W8, 3>(p, t);
+  else
+    splitk_reduce_add_rmsnorm_body<TPR, MAXC, W8, 7>(p, t);
 }
 
 // ---------------------------------------------------------------------------
