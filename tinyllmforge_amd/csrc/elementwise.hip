@@ -31,18 +31,26 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(
 
   float v[MAXC][8];
   uint4 pw[MAXC];  // the weights do not depend on the row: fetched together with it, not after the reduction
+  uint4 px[MAXC], pres[MAXC];
+  // every load of the row is unconditional (a chunk past the row re-reads the row's last chunk, an idle thread row 0)
+  // and stands before the first use, so that all of them are in flight at once; only the arithmetic and the stores
+  // are predicated
+#pragma unroll
+  for (int c = 0; c < MAXC; ++c) {
+    const int at = min(sub + c * TPR, nchunks - 1) * 8;
+    pw[c] = *reinterpret_cast<const uint4 *>(weight + at);
+    px[c] = *reinterpret_cast<const uint4 *>(xr + at);
+    if (ADD) pres[c] = *reinterpret_cast<const uint4 *>(residual + out_off + at);
+  }
   float ss = 0.f;
 #pragma unroll
   for (int c = 0; c < MAXC; ++c) {
     const int chunk = sub + c * TPR;
-    pw[c] = make_uint4(0, 0, 0, 0);
     if (active && chunk < nchunks) {
-      pw[c] = *reinterpret_cast<const uint4 *>(weight + chunk * 8);
-      uint4 p = *reinterpret_cast<const uint4 *>(xr + chunk * 8);
-      unpack8(p, v[c]);
+      unpack8(px[c], v[c]);
       if (ADD) {
         float r[8];
-        uint4 pr = *reinterpret_cast<const uint4 *>(residual + out_off + chunk * 8);
+        const uint4 pr = pres[c];
         unpack8(pr, r);
 #pragma unroll
         for (int i = 0; i < 8; ++i) v[c][i] = __fadd_rn(v[c][i], r[i]);
