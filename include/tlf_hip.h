@@ -371,6 +371,31 @@ int tlf_paged_decode_attn(const void *q, int64_t q_stride,
                           int64_t num_cache_blocks, float scale,
                           void *workspace, size_t workspace_bytes, void *stream);
 
+/* a3 with the split of the work made once per decode step instead of once per layer (build-defined; the reference
+ * calls flash_attn_with_kvcache per layer, layers/attention.py:106-109, and every layer of a step passes the same
+ * context_lens and block_tables).  tlf_paged_decode_plan scans the lengths, finds every workgroup's first sequence
+ * and copies the block-table entries it needs first into plan (tlf_paged_decode_plan_bytes() bytes, 16-byte
+ * aligned); tlf_paged_decode_attn_planned is tlf_paged_decode_attn reading that plan: same arguments (the lengths
+ * and tables must be the ones the plan was made from, with the same batch, block_size and max_blocks), same
+ * results bit for bit, and its first cache rows are requested one memory round trip after the kernel starts
+ * instead of three.  The plan is read-only to the attention calls: one plan serves all layers of the step.  A plan
+ * made for another batch size (or for a grid another max_blocks / block_size gives) is recognised by its header
+ * and turns every output row into NaN; one made from other lengths of the same batch cannot be told apart and gives
+ * what those lengths would give. */
+size_t tlf_paged_decode_plan_bytes(void);
+int tlf_paged_decode_plan(const int32_t *context_lens, const int32_t *block_tables,
+                          int64_t block_table_stride, int32_t batch, int32_t block_size,
+                          int32_t max_blocks, void *plan, size_t plan_bytes, void *stream);
+int tlf_paged_decode_attn_planned(const void *q, int64_t q_stride,
+                                  const void *k_cache, const void *v_cache, int32_t kv_dtype,
+                                  const float *k_scale, const float *v_scale,
+                                  const int32_t *block_tables, int64_t block_table_stride,
+                                  const int32_t *context_lens, void *out,
+                                  int32_t batch, int32_t num_q_heads, int32_t num_kv_heads,
+                                  int32_t head_dim, int32_t block_size, int32_t max_blocks,
+                                  int64_t num_cache_blocks, float scale,
+                                  void *workspace, size_t workspace_bytes, const void *plan, void *stream);
+
 /* ---------------------------------------------------------------------------
  * a4  varlen causal prefill attention   replaces the prefill branch
  *     layers/attention.py:96-105 (flash_attn_varlen_func, causal=True)

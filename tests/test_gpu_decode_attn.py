@@ -31,7 +31,12 @@ def run_both(case, scale=128 ** -0.5):
     from tinyllmforge_amd import ops as P
     q, kc, vc, cl, bt = case
     ref = O.paged_decode_attention(q, kc, vc, cl, bt, scale)
-    got = P.paged_decode_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), cl.to(DEV), bt.to(DEV), scale).cpu()
+    dq, dk, dv, dcl, dbt = q.to(DEV), kc.to(DEV), vc.to(DEV), cl.to(DEV), bt.to(DEV)
+    got = P.paged_decode_attention(dq, dk, dv, dcl, dbt, scale).cpu()
+    # the same call with the work split made beforehand (once per decode step in the engine): same bits
+    plan = P.paged_decode_plan(dcl, dbt, kc.shape[1])
+    planned = P.paged_decode_attention(dq, dk, dv, dcl, dbt, scale, plan=plan).cpu()
+    assert torch.equal(planned.view(torch.int16), got.view(torch.int16)), "planned call differs"
     return got, ref
 
 
@@ -161,8 +166,11 @@ def _run_fp8(case, scale=0.0884):
     from tinyllmforge_amd import ops as P
     q, k8, v8, cl, bt, ks, vs = case
     ref = O.paged_decode_attention(q, k8, v8, cl, bt, scale, ks, vs)
-    got = P.paged_decode_attention(q.to(DEV), k8.to(DEV), v8.to(DEV), cl.to(DEV), bt.to(DEV), scale,
-                                   ks.to(DEV), vs.to(DEV)).cpu()
+    dev = [t.to(DEV) for t in (q, k8, v8, cl, bt)]
+    got = P.paged_decode_attention(*dev, scale, ks.to(DEV), vs.to(DEV)).cpu()
+    plan = P.paged_decode_plan(dev[3], dev[4], k8.shape[1])
+    planned = P.paged_decode_attention(*dev, scale, ks.to(DEV), vs.to(DEV), plan=plan).cpu()
+    assert torch.equal(planned.view(torch.int16), got.view(torch.int16)), "planned call differs"
     return got, ref
 
 
@@ -213,3 +221,48 @@ def test_decode_segment_changes_inside_a_workgroup_bf16():
     ctxs[200] = 0
     got, ref = run_both(make_case(37, len(ctxs), 32, 8, 16, ctxs, sum((c + 15) // 16 for c in ctxs) + 2))
     check(got, ref)
+
+
+def test_one_plan_serves_every_layer_of_a_step():
+    """The engine makes the plan once per decode step: the same plan with other queries and other caches (another
+    layer) gives that layer's unplanned result bit for bit, also after the plan buffer was re-used for another
+    step (other lengths) and made again; the plan holds what the kernel's own scan would find (header, prefix sums
+    and the first sequence of every workgroup's share)."""
+    from tinyllmforge_amd import ops as P
+    ge = torch.Generator().manual_seed(3)
+    ctxs = torch.randint(1, 3000, (40,), generator=ge).tolist()
+    ctxs[5] = 0
+    layers = [make_case(50 + i, len(ctxs), 32, 8, 256, ctxs, 300, maxb=16) for i in range(3)]
+    cl, bt = layers[0][3].to(DEV), layers[0][4].to(DEV)
+    plan = P.paged_decode_plan(cl, bt, 256)
+    hdr = plan[:4].tolist()
+    tiles = [(c + 15) // 16 for c in ctxs]
+    assert hdr[0] == sum(tiles) and hdr[3] == len(ctxs) and hdr[1] == max(4, -(-hdr[0] // hdr[2]))
+    prefix = plan[16:16 + len(ctxs) + 1].tolist()
+    assert prefix == [sum(tiles[:i]) for i in range(len(ctxs) + 1)]
+    rec0 = 16 + 1024 + 16 + 1024
+    for wg in (0, 1, hdr[2] // 2, hdr[2] - 1):
+        b, first, end, length = plan[rec0 + 72 * wg: rec0 + 72 * wg + 4].tolist()
+        ts = wg * hdr[1]
+        if ts < hdr[0]:
+            assert first <= ts < end and (first, end, length) == (prefix[b], prefix[b + 1], ctxs[b])
+            base = (ts - first) * 16 // 256
+            want = [int(bt[b, min(base + l, 15)]) for l in range(64)]
+            assert plan[rec0 + 72 * wg + 8: rec0 + 72 * wg + 72].tolist() == want
+        else:
+            assert b == -1
+    for q, kc, vc, _, _ in layers:       # the tables are layer 0's: a layer differs in q and in its cache
+        a = P.paged_decode_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), cl, bt, 0.0884)
+        b = P.paged_decode_attention(q.to(DEV), kc.to(DEV), vc.to(DEV), cl, bt, 0.0884, plan=plan)
+        assert torch.equal(a, b)
+    other = torch.tensor([7] * len(ctxs), dtype=torch.int32, device=DEV)
+    P.paged_decode_plan(other, bt, 256, out=plan)
+    short = P.paged_decode_attention(layers[0][0].to(DEV), layers[0][1].to(DEV), layers[0][2].to(DEV), other, bt, 0.0884, plan=plan)
+    assert torch.equal(short, P.paged_decode_attention(layers[0][0].to(DEV), layers[0][1].to(DEV), layers[0][2].to(DEV), other, bt, 0.0884))
+    P.paged_decode_plan(cl, bt, 256, out=plan)
+    q, kc, vc = (t.to(DEV) for t in layers[1][:3])
+    assert torch.equal(P.paged_decode_attention(q, kc, vc, cl, bt, 0.0884, plan=plan), P.paged_decode_attention(q, kc, vc, cl, bt, 0.0884))
+    # a plan made for another batch size is recognised and refused loudly
+    few = P.paged_decode_plan(cl[:7].contiguous(), bt[:7].contiguous(), 256)
+    bad = P.paged_decode_attention(q, kc, vc, cl, bt, 0.0884, plan=few)
+    assert torch.isnan(bad.float()).all()

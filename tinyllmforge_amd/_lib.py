@@ -58,6 +58,10 @@ SIGNATURES = {
     "tlf_paged_decode_attn_workspace_bytes": (_SZ, [_I32, _I32, _I32, _I32, _I32]),
     "tlf_paged_decode_attn": (c_int32, [_P, _I64, _P, _P, _I32, _P, _P, _P, _I64, _P, _P,
                                         _I32, _I32, _I32, _I32, _I32, _I32, _I64, _F, _P, _SZ, _P]),
+    "tlf_paged_decode_plan_bytes": (_SZ, []),
+    "tlf_paged_decode_plan": (c_int32, [_P, _P, _I64, _I32, _I32, _I32, _P, _SZ, _P]),
+    "tlf_paged_decode_attn_planned": (c_int32, [_P, _I64, _P, _P, _I32, _P, _P, _P, _I64, _P, _P,
+                                                _I32, _I32, _I32, _I32, _I32, _I32, _I64, _F, _P, _SZ, _P, _P]),
     "tlf_varlen_prefill_attn": (c_int32, [_P, _I64, _P, _I64, _P, _I64, _I32, _P, _P, _P, _P, _P, _I64,
                                           _P, _I32, _I32, _I32, _I32, _I32, _I32, _I64, _F, _P]),
     "tlf_embedding": (c_int32, [_P, _P, _P, _I32, _I32, _I32, _P]),

@@ -89,6 +89,9 @@ class Config:
     # keeps two steps in flight and patches the values into its sequences as they arrive.  Same tokens, same
     # block ids and step counts as the step-by-step loop; False restores that loop.
     run_ahead: bool = True
+    # The decode attention kernel's split of the step's work over the workgroups is made once per step (one small
+    # kernel at the head of the step) instead of by every layer's call: same results, a shorter start per layer.
+    decode_plan: bool = True
 
     def __post_init__(self):
         if isinstance(self.model, str) and self.model.lower() in QWEN3_SHAPES:

@@ -72,7 +72,17 @@ struct DecodeParams {
   int32_t max_blocks;
   int64_t num_cache_blocks;
   float scale_log2;  // softmax scale * log2(e)
+  const int32_t *plan;  // null, or the output of plan_decode_kernel for these lengths, tables and this grid
 };
+
+// Layout of a plan (int32): header {total tiles, tiles per workgroup, grid, batch}, the prefix table, the clamped
+// lengths, then one record per workgroup: {first sequence, its first tile, its end tile, its length, 0 ...} and the
+// 64 block-table entries a wave holds for that sequence from the share's first block on.
+constexpr int kPlanPrefix = 16;
+constexpr int kPlanCtx = kPlanPrefix + kMaxBatch + 16;
+constexpr int kPlanRec = kPlanCtx + kMaxBatch;
+constexpr int kPlanRecInts = 8 + 64;
+constexpr int kPlanInts = kPlanRec + kMaxGrid * kPlanRecInts;
 
 __device__ __forceinline__ shortx4 lds_read_tr16_b64(const unsigned short *p) {
   // within each group of 16 lanes, lane i receives {row0[i], row1[i], row2[i], row3[i]},
@@ -141,57 +151,6 @@ void paged_decode_kernel(const DecodeParams p) {
   const float kscale = KV8 ? p.k_scale[w] : 1.0f;
   const float vscale = KV8 ? p.v_scale[w] : 1.0f;
 
-  // ---- 1. tiles per sequence -> exclusive prefix in LDS (block scan, chunks of kThreads)
-  if (tid == 0) s_prefix[0] = 0;
-  int carry = 0;
-  for (int base = 0; base < p.batch; base += kThreads) {
-    const int b = base + tid;
-    int tiles = 0;
-    if (b < p.batch) {
-      const int c = min(p.context_lens[b], max_ctx);
-      s_ctx[b] = c;
-      tiles = c > 0 ? (c + kTile - 1) / kTile : 0;
-    }
-    int incl = tiles;
-#pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-      const int up = __shfl_up(incl, o, 64);
-      if (lane >= o) incl += up;
-    }
-    if (lane == 63) s_wave_tot[w] = incl;
-    __syncthreads();
-    int before = carry;
-    for (int ww = 0; ww < w; ++ww) before += s_wave_tot[ww];
-    if (b < p.batch) s_prefix[b + 1] = before + incl;
-    int total = 0;
-    for (int ww = 0; ww < NW; ++ww) total += s_wave_tot[ww];
-    carry += total;
-    __syncthreads();
-  }
-  const int total_tiles = carry;
-
-  // ---- 2. empty sequences get zeros: workgroup i looks after sequences i, i + G, ... (one workgroup walking
-  // the whole batch would finish its own share that much later, and the launch with it)
-  for (int b = blockIdx.x; b < p.batch; b += gridDim.x) {
-    if (s_prefix[b + 1] == s_prefix[b]) {
-      if (tid == 0) *reinterpret_cast<int2 *>(p.meta + 2 * b) = make_int2(0, 0);
-      unsigned short *o = p.out + static_cast<int64_t>(b) * p.num_q_heads * kDh;
-      for (int i = tid * 8; i < p.num_q_heads * kDh; i += kThreads * 8)
-        *reinterpret_cast<uint4 *>(o + i) = make_uint4(0, 0, 0, 0);
-    }
-  }
-
-  // ---- 3. this workgroup's share [ts, te) of the flat tile list
-  const int G = gridDim.x;
-  int tpw = (total_tiles + G - 1) / G;
-  if (tpw < kMinTiles) tpw = kMinTiles;
-  const int ts = blockIdx.x * tpw;
-  const int te = min(total_tiles, ts + tpw);
-  if (ts >= total_tiles) return;  // uniform
-  for (int b = tid; b < p.batch; b += kThreads)
-    if (s_prefix[b] <= ts && ts < s_prefix[b + 1]) s_start_b = b;
-  __syncthreads();
-
   const int64_t row_elems = static_cast<int64_t>(p.num_kv_heads) * kDh;
   unsigned short(*Ks)[kLdsRowK] = lds_k[w];
   unsigned short(*Vs)[kLdsRowV] = lds_v[w];
@@ -221,7 +180,7 @@ void paged_decode_kernel(const DecodeParams p) {
     bf16x8 qf[4];
     int bt_vec, bt_base;
   };
-  auto fetch_seg = [&](int sb, int t_begin, SegRegs &r) {
+  auto fetch_q = [&](int sb, SegRegs &r) {
     const unsigned short *qp = p.q + sb * p.q_stride + static_cast<int64_t>(head) * kDh;
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
@@ -230,8 +189,23 @@ void paged_decode_kernel(const DecodeParams p) {
       if (head_ok) t.u = *reinterpret_cast<const uint4 *>(qp + lds_col_dim<KV8>(c * 32 + g * 8));
       r.qf[c] = t.v;
     }
+  };
+  auto fetch_seg = [&](int sb, int t_begin, SegRegs &r) {
+    fetch_q(sb, r);
     r.bt_base = t_begin / p.block_size;
     r.bt_vec = (p.block_tables + sb * p.bt_stride)[min(r.bt_base + lane, p.max_blocks - 1)];
+  };
+  // empty sequences get zeros: workgroup i looks after sequences i, i + G, ... (one workgroup walking the whole
+  // batch would finish its own share that much later, and the launch with it)
+  auto zero_empty = [&]() {
+    for (int b = blockIdx.x; b < p.batch; b += gridDim.x) {
+      if (s_prefix[b + 1] == s_prefix[b]) {
+        if (tid == 0) *reinterpret_cast<int2 *>(p.meta + 2 * b) = make_int2(0, 0);
+        unsigned short *o = p.out + static_cast<int64_t>(b) * p.num_q_heads * kDh;
+        for (int i = tid * 8; i < p.num_q_heads * kDh; i += kThreads * 8)
+          *reinterpret_cast<uint4 *>(o + i) = make_uint4(0, 0, 0, 0);
+      }
+    }
   };
 
   // Issue the loads of the tile starting at token t0 (a tile never straddles a block); blk is its
@@ -306,17 +280,118 @@ void paged_decode_kernel(const DecodeParams p) {
   };
 
 
+  int total_tiles, tpw, ts, te;
+  TLF_SEG_DECL(sg_);
+  TLF_SEG_DECL(sn_);
+  SegRegs cur_regs, next_regs;
+  if (p.plan == nullptr) {
+  // ---- 1. tiles per sequence -> exclusive prefix in LDS (block scan, chunks of kThreads)
+  if (tid == 0) s_prefix[0] = 0;
+  int carry = 0;
+  for (int base = 0; base < p.batch; base += kThreads) {
+    const int b = base + tid;
+    int tiles = 0;
+    if (b < p.batch) {
+      const int c = min(p.context_lens[b], max_ctx);
+      s_ctx[b] = c;
+      tiles = c > 0 ? (c + kTile - 1) / kTile : 0;
+    }
+    int incl = tiles;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += up;
+    }
+    if (lane == 63) s_wave_tot[w] = incl;
+    __syncthreads();
+    int before = carry;
+    for (int ww = 0; ww < w; ++ww) before += s_wave_tot[ww];
+    if (b < p.batch) s_prefix[b + 1] = before + incl;
+    int total = 0;
+    for (int ww = 0; ww < NW; ++ww) total += s_wave_tot[ww];
+    carry += total;
+    __syncthreads();
+  }
+  total_tiles = carry;
+
+  // ---- 2. empty sequences get zeros
+  zero_empty();
+
+  // ---- 3. this workgroup's share [ts, te) of the flat tile list
+  const int G = gridDim.x;
+  tpw = (total_tiles + G - 1) / G;
+  if (tpw < kMinTiles) tpw = kMinTiles;
+  ts = blockIdx.x * tpw;
+  te = min(total_tiles, ts + tpw);
+  if (ts >= total_tiles) return;  // uniform
+  for (int b = tid; b < p.batch; b += kThreads)
+    if (s_prefix[b] <= ts && ts < s_prefix[b + 1]) s_start_b = b;
+  __syncthreads();
+
   // One trip is in flight per wave (deeper register prefetch was measured and is no faster: the stream is not
   // bound by this wave's latency once every CU has 64 KB in flight).  What is pipelined is the change of
   // segment: q and the block-table entries of the next segment are fetched while the current one runs, and the
   // first trip of the next segment is loaded during the last trip of the current one, so a workgroup whose
   // share covers several sequences does not stop streaming between them.
-  TLF_SEG_DECL(sg_);
-  TLF_SEG_DECL(sn_);
   TLF_SEG_MAKE(sg_, ts, s_start_b)
-  SegRegs cur_regs, next_regs;
   fetch_seg(sg_b, sg_t_begin, next_regs);
   load_trip(sg_t_begin, sg_t_end, next_regs.bt_vec, next_regs.bt_base);
+  } else {
+    // ---- the same three steps from a plan made once per decode step (plan_decode_kernel) instead of once per
+    // layer: the prefix table and the lengths are copied, and the record of this workgroup names its first sequence
+    // and holds that sequence's block-table entries, so the first rows are requested one memory round trip after
+    // the kernel starts instead of three (lengths -> scan and search -> block table -> rows).
+    const int32_t *pl = p.plan;
+    const int4 hdr = *reinterpret_cast<const int4 *>(pl);   // total tiles, tiles per workgroup, grid, batch
+    const int32_t *recp = pl + kPlanRec + static_cast<int64_t>(blockIdx.x) * kPlanRecInts;
+    const int4 rec = *reinterpret_cast<const int4 *>(recp);  // first sequence of the share, its tiles [first, end), its length
+    const int bt_first = recp[8 + lane];
+    constexpr int kCopies = kMaxBatch / kThreads + 1;
+    int cp[kCopies], cc[kCopies];
+#pragma unroll
+    for (int i = 0; i < kCopies; ++i) {
+      const int b = min(tid + i * kThreads, p.batch);
+      cp[i] = pl[kPlanPrefix + b];
+      cc[i] = pl[kPlanCtx + min(b, p.batch - 1)];
+    }
+    if (hdr.z != static_cast<int>(gridDim.x) || hdr.w != p.batch || hdr.y < kMinTiles) {
+      // a plan made for another grid or batch: nothing of it can be trusted; every output row becomes NaN
+      for (int b = blockIdx.x; b < p.batch; b += gridDim.x) {
+        unsigned short *o = p.out + static_cast<int64_t>(b) * p.num_q_heads * kDh;
+        for (int i = tid * 8; i < p.num_q_heads * kDh; i += kThreads * 8)
+          *reinterpret_cast<uint4 *>(o + i) = make_uint4(0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u, 0x7fc07fc0u);
+        if (tid == 0) *reinterpret_cast<int2 *>(p.meta + 2 * b) = make_int2(0, 0);
+      }
+      return;
+    }
+    total_tiles = __builtin_amdgcn_readfirstlane(hdr.x);
+    tpw = __builtin_amdgcn_readfirstlane(hdr.y);
+    ts = blockIdx.x * tpw;
+    te = min(total_tiles, ts + tpw);
+    const bool has_work = ts < total_tiles;
+    if (has_work) {
+      sg_b = __builtin_amdgcn_readfirstlane(rec.x);
+      sg_seq_first = __builtin_amdgcn_readfirstlane(rec.y);
+      sg_seq_end = __builtin_amdgcn_readfirstlane(rec.z);
+      const int seg_end_ = min(te, sg_seq_end);
+      sg_t_begin = (ts - sg_seq_first) * kTile;
+      sg_t_end = min(__builtin_amdgcn_readfirstlane(rec.w), (seg_end_ - sg_seq_first) * kTile);
+      sg_last = seg_end_ >= te;
+      fetch_q(sg_b, next_regs);
+      next_regs.bt_base = sg_t_begin / p.block_size;
+      next_regs.bt_vec = bt_first;
+      load_trip(sg_t_begin, sg_t_end, next_regs.bt_vec, next_regs.bt_base);
+    }
+#pragma unroll
+    for (int i = 0; i < kCopies; ++i) {
+      const int b = tid + i * kThreads;
+      if (b <= p.batch) s_prefix[b] = cp[i];
+      if (b < p.batch) s_ctx[b] = cc[i];
+    }
+    __syncthreads();
+    zero_empty();
+    if (!has_work) return;  // uniform
+  }
   while (true) {
     cur_regs = next_regs;
     sn_b = sg_b; sn_seq_first = sg_seq_first; sn_seq_end = sg_seq_end; sn_t_begin = 0; sn_t_end = 0; sn_last = 1;
@@ -543,6 +618,81 @@ __global__ __launch_bounds__(256) void paged_decode_merge_kernel(const DecodePar
   *reinterpret_cast<uint2 *>(p.out + (static_cast<int64_t>(b) * p.num_q_heads + hh) * kDh + c4) = st;
 }
 
+// The work split of paged_decode_kernel, made once per decode step for all layers (their lengths and block tables
+// are the same).  Every workgroup scans the lengths as step 1 of that kernel does (1024 threads, one chunk), then
+// writes the records of 16 of the G attention workgroups: 16 threads find their first sequences, all 1024 copy the
+// 64 block-table entries of each; workgroup 0 also writes the header, the prefix table and the lengths.
+constexpr int kPlanRecsPerWg = 16;
+__global__ __launch_bounds__(1024) void plan_decode_kernel(const int32_t *__restrict__ context_lens,
+                                                           const int32_t *__restrict__ block_tables, int64_t bt_stride,
+                                                           int32_t batch, int32_t block_size, int32_t max_blocks, int32_t G,
+                                                           int32_t *__restrict__ plan) {
+  __shared__ int s_prefix[kMaxBatch + 1];
+  __shared__ int s_ctx[kMaxBatch];
+  __shared__ int s_wave_tot[16];
+  __shared__ int s_rec_b[kPlanRecsPerWg];
+  const int tid = threadIdx.x, w = tid >> 6, lane = tid & 63;
+  const int max_ctx = max_blocks * block_size;
+  int tiles = 0;
+  if (tid < batch) {
+    const int c = min(context_lens[tid], max_ctx);
+    s_ctx[tid] = c;
+    tiles = c > 0 ? (c + kTile - 1) / kTile : 0;
+  }
+  int incl = tiles;
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int up = __shfl_up(incl, o, 64);
+    if (lane >= o) incl += up;
+  }
+  if (lane == 63) s_wave_tot[w] = incl;
+  if (tid == 0) s_prefix[0] = 0;
+  __syncthreads();
+  int before = 0, total = 0;
+  for (int ww = 0; ww < 16; ++ww) {
+    if (ww < w) before += s_wave_tot[ww];
+    total += s_wave_tot[ww];
+  }
+  if (tid < batch) s_prefix[tid + 1] = before + incl;
+  __syncthreads();
+  int tpw = (total + G - 1) / G;
+  if (tpw < kMinTiles) tpw = kMinTiles;
+  if (blockIdx.x == 0) {
+    if (tid == 0) *reinterpret_cast<int4 *>(plan) = make_int4(total, tpw, G, batch);
+    for (int b = tid; b <= batch; b += 1024) plan[kPlanPrefix + b] = s_prefix[b];
+    if (tid < batch) plan[kPlanCtx + tid] = s_ctx[tid];
+  }
+  const int i0 = blockIdx.x * kPlanRecsPerWg;
+  if (tid < kPlanRecsPerWg && i0 + tid < G) {
+    const int i = i0 + tid;
+    const int ts = i * tpw;
+    int b = -1;
+    if (ts < total) {  // the sequence whose tiles [prefix[b], prefix[b + 1]) hold tile ts (never an empty one)
+      int lo = 0, hi = batch - 1;
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (s_prefix[mid + 1] > ts) hi = mid; else lo = mid + 1;
+      }
+      b = lo;
+    }
+    s_rec_b[tid] = b;
+    int32_t *rec = plan + kPlanRec + static_cast<int64_t>(i) * kPlanRecInts;
+    *reinterpret_cast<int4 *>(rec) = b >= 0 ? make_int4(b, s_prefix[b], s_prefix[b + 1], s_ctx[b]) : make_int4(-1, 0, 0, 0);
+    *reinterpret_cast<int4 *>(rec + 4) = make_int4(0, 0, 0, 0);
+  }
+  __syncthreads();
+  const int i = i0 + w;   // wave w copies the entries of record i0 + w
+  if (i < G) {
+    const int b = s_rec_b[w];
+    int v = -1;
+    if (b >= 0) {
+      const int bt_base = (i * tpw - s_prefix[b]) * kTile / block_size;
+      v = block_tables[b * bt_stride + min(bt_base + lane, max_blocks - 1)];
+    }
+    plan[kPlanRec + static_cast<int64_t>(i) * kPlanRecInts + 8 + lane] = v;
+  }
+}
+
 inline int device_cu_count() {
   static int cus = 0;
   if (cus == 0) {
@@ -588,14 +738,44 @@ extern "C" size_t tlf_paged_decode_attn_workspace_bytes(int32_t batch, int32_t n
          slots * num_q_heads * (static_cast<size_t>(head_dim) + 2) * sizeof(float);
 }
 
-extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void *k_cache,
+namespace tlf {
+// persistent grid: one workgroup per CU (decode_wgs_per_cu), fewer when the largest possible job is small
+inline int decode_grid(int32_t batch, int32_t max_blocks, int32_t block_size) {
+  const int64_t max_tiles = static_cast<int64_t>(batch) * ((static_cast<int64_t>(max_blocks) * block_size + kTile - 1) / kTile);
+  int64_t grid = static_cast<int64_t>(decode_wgs_per_cu()) * device_cu_count();
+  if (grid > kMaxGrid) grid = kMaxGrid;
+  const int64_t by_work = (max_tiles + kMinTiles - 1) / kMinTiles;
+  if (grid > by_work) grid = by_work;
+  if (grid < 1) grid = 1;
+  return static_cast<int>(grid);
+}
+}  // namespace tlf
+
+extern "C" size_t tlf_paged_decode_plan_bytes(void) { return static_cast<size_t>(kPlanInts) * sizeof(int32_t); }
+
+extern "C" int tlf_paged_decode_plan(const int32_t *context_lens, const int32_t *block_tables,
+                                     int64_t block_table_stride, int32_t batch, int32_t block_size,
+                                     int32_t max_blocks, void *plan, size_t plan_bytes, void *stream) {
+  if (batch == 0) return TLF_OK;
+  if (!context_lens || !block_tables || !plan) return TLF_E_NULL;
+  if (batch < 0 || batch > kMaxBatch || block_size <= 0 || max_blocks <= 0 || block_size % kTile) return TLF_E_SHAPE;
+  if (static_cast<int64_t>(max_blocks) * block_size > (1ll << 30) || block_table_stride < max_blocks) return TLF_E_SHAPE;
+  if (plan_bytes < tlf_paged_decode_plan_bytes() || !aligned16(plan)) return TLF_E_WORKSPACE;
+  const int grid = decode_grid(batch, max_blocks, block_size);
+  TLF_LAUNCH(plan_decode_kernel, dim3((grid + kPlanRecsPerWg - 1) / kPlanRecsPerWg), dim3(1024), 0,
+             static_cast<hipStream_t>(stream), context_lens, block_tables, block_table_stride, batch, block_size,
+             max_blocks, grid, static_cast<int32_t *>(plan));
+  return launch_status();
+}
+
+static int decode_attn_impl(const void *q, int64_t q_stride, const void *k_cache,
                                      const void *v_cache, int32_t kv_dtype, const float *k_scale,
                                      const float *v_scale, const int32_t *block_tables,
                                      int64_t block_table_stride, const int32_t *context_lens,
                                      void *out, int32_t batch, int32_t num_q_heads,
                                      int32_t num_kv_heads, int32_t head_dim, int32_t block_size,
                                      int32_t max_blocks, int64_t num_cache_blocks, float scale,
-                                     void *workspace, size_t workspace_bytes, void *stream) {
+                                     void *workspace, size_t workspace_bytes, const int32_t *plan, void *stream) {
   if (batch == 0) return TLF_OK;
   if (!q || !k_cache || !v_cache || !block_tables || !context_lens || !out) return TLF_E_NULL;
   if (head_dim != kDh) return TLF_E_UNSUPPORTED;
@@ -641,13 +821,8 @@ extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void
   p.part_ml = reinterpret_cast<float *>(ws + decode_meta_bytes());
   p.part_o = p.part_ml + slots * num_q_heads * 2;
 
-  // persistent grid: one workgroup per CU (decode_wgs_per_cu), fewer when the largest possible job is small
-  const int64_t max_tiles = static_cast<int64_t>(batch) * ((static_cast<int64_t>(max_blocks) * block_size + kTile - 1) / kTile);
-  int64_t grid = static_cast<int64_t>(decode_wgs_per_cu()) * device_cu_count();
-  if (grid > kMaxGrid) grid = kMaxGrid;
-  const int64_t by_work = (max_tiles + kMinTiles - 1) / kMinTiles;
-  if (grid > by_work) grid = by_work;
-  if (grid < 1) grid = 1;
+  p.plan = plan;
+  const int grid = decode_grid(batch, max_blocks, block_size);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 g(static_cast<unsigned>(grid));
   const bool f8 = kv_dtype == TLF_KV_FP8_E4M3;
@@ -670,4 +845,31 @@ extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void
   if (rc != TLF_OK) return rc;
   TLF_LAUNCH(paged_decode_merge_kernel, dim3((num_q_heads + 7) / 8, batch), dim3(256), 0, s, p);
   return launch_status();
+}
+
+extern "C" int tlf_paged_decode_attn(const void *q, int64_t q_stride, const void *k_cache,
+                                     const void *v_cache, int32_t kv_dtype, const float *k_scale,
+                                     const float *v_scale, const int32_t *block_tables,
+                                     int64_t block_table_stride, const int32_t *context_lens,
+                                     void *out, int32_t batch, int32_t num_q_heads,
+                                     int32_t num_kv_heads, int32_t head_dim, int32_t block_size,
+                                     int32_t max_blocks, int64_t num_cache_blocks, float scale,
+                                     void *workspace, size_t workspace_bytes, void *stream) {
+  return decode_attn_impl(q, q_stride, k_cache, v_cache, kv_dtype, k_scale, v_scale, block_tables, block_table_stride,
+                          context_lens, out, batch, num_q_heads, num_kv_heads, head_dim, block_size, max_blocks,
+                          num_cache_blocks, scale, workspace, workspace_bytes, nullptr, stream);
+}
+
+extern "C" int tlf_paged_decode_attn_planned(const void *q, int64_t q_stride, const void *k_cache,
+                                             const void *v_cache, int32_t kv_dtype, const float *k_scale,
+                                             const float *v_scale, const int32_t *block_tables,
+                                             int64_t block_table_stride, const int32_t *context_lens,
+                                             void *out, int32_t batch, int32_t num_q_heads,
+                                             int32_t num_kv_heads, int32_t head_dim, int32_t block_size,
+                                             int32_t max_blocks, int64_t num_cache_blocks, float scale,
+                                             void *workspace, size_t workspace_bytes, const void *plan, void *stream) {
+  if (batch != 0 && (!plan || !aligned16(plan))) return plan ? TLF_E_ALIGN : TLF_E_NULL;
+  return decode_attn_impl(q, q_stride, k_cache, v_cache, kv_dtype, k_scale, v_scale, block_tables, block_table_stride,
+                          context_lens, out, batch, num_q_heads, num_kv_heads, head_dim, block_size, max_blocks,
+                          num_cache_blocks, scale, workspace, workspace_bytes, static_cast<const int32_t *>(plan), stream);
 }

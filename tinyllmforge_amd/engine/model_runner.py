@@ -11,7 +11,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 
-from .. import _lib
+from .. import _lib, ops
 from ..config import Config
 from ..layers.sampler import Sampler
 from ..models.qwen3 import Qwen3ForCausalLM
@@ -229,6 +229,8 @@ class ModelRunner:
         ctx = get_context()
         if (is_prefill or self.enforce_eager or not self.graph_bs or bs > self.graph_bs[-1]
                 or ctx.block_tables is None or ctx.block_tables.size(1) > self.graph_max_blocks):
+            if not is_prefill:
+                self.plan_decode()
             return self.model(input_ids, positions)      # a table wider than the graphs' static one runs eagerly
         gbs = next(x for x in self.graph_bs if x >= bs)
         gv = self.graph_vars
@@ -245,6 +247,16 @@ class ModelRunner:
         gv["block_tables"][:bs, :w] = ctx.block_tables
         self.graphs[gbs].replay()
         return gv["outputs"][:bs]
+
+    def plan_decode(self):
+        """The attention kernel's work split of this decode step, made once for all layers (they share the
+        lengths and the block tables) into one buffer that every step and every captured graph re-uses."""
+        ctx = get_context()
+        if (not self.config.decode_plan or ctx.context_lens is None or ctx.block_tables is None
+                or ctx.context_lens.numel() > 1024):
+            return      # switched off, or more sequences than a plan holds: every layer scans for itself
+        ctx.decode_plan = self.decode_plan_buf = ops.paged_decode_plan(ctx.context_lens, ctx.block_tables, self.block_size,
+                                                                       out=getattr(self, "decode_plan_buf", None))
 
     @torch.inference_mode()
     def run_model(self, input_ids, positions, is_prefill):
@@ -393,9 +405,11 @@ class ModelRunner:
             graph = torch.cuda.CUDAGraph()
             set_context(False, slot_mapping=gv["slot_mapping"][:bs], context_lens=gv["context_lens"][:bs],
                         block_tables=gv["block_tables"][:bs, :])
+            self.plan_decode()
             gv["outputs"][:bs] = self.model(gv["input_ids"][:bs], gv["positions"][:bs])    # warm-up
             launched = lib.tlf_kernel_launches()
             with torch.cuda.graph(graph, pool):
+                self.plan_decode()       # first node of the graph: the attention work split of the step
                 gv["outputs"][:bs] = self.model(gv["input_ids"][:bs], gv["positions"][:bs])
             self.graph_kernels[bs] = lib.tlf_kernel_launches() - launched + 1    # + the copy into the static output
             if pool is None:

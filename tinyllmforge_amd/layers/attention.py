@@ -44,4 +44,4 @@ class Attention(nn.Module):
                                                 v.view(-1, self.num_kv_heads, self.head_dim),
                                                 ctx.cu_seqlens_q, ctx.cu_seqlens_k, ctx.max_seqlen_q, self.scale)
         return ops.paged_decode_attention(q, self.k_cache, self.v_cache, ctx.context_lens, ctx.block_tables,
-                                          self.scale, self.k_scale, self.v_scale)
+                                          self.scale, self.k_scale, self.v_scale, plan=ctx.decode_plan)

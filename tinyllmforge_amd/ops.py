@@ -402,9 +402,26 @@ def linear_qknorm_rope_store(x, w, scale, q_weight, k_weight, eps, positions, co
 
 
 # ------------------------------------------------------------------ a3
+def paged_decode_plan(context_lens, block_tables, block_size, out=None):
+    """The work split of ``paged_decode_attention`` for one decode step, made once for all layers (they share the
+    lengths and the block tables).  Returns an int32 tensor to pass as ``plan=``; ``out`` re-uses one (a captured
+    graph keeps its pointer)."""
+    lib = _lib.load()
+    _need(context_lens, torch.int32, "context_lens"); _need(block_tables, torch.int32, "block_tables")
+    assert block_tables.stride(1) == 1 and context_lens.is_contiguous()
+    nbytes = lib.tlf_paged_decode_plan_bytes()
+    plan = out if out is not None else torch.empty(nbytes // 4, dtype=torch.int32, device=context_lens.device)
+    assert plan.dtype == torch.int32 and plan.numel() * 4 >= nbytes and plan.is_contiguous()
+    check(lib.tlf_paged_decode_plan(context_lens.data_ptr(), block_tables.data_ptr(), block_tables.stride(0),
+                                    context_lens.numel(), int(block_size), block_tables.shape[1], plan.data_ptr(),
+                                    plan.numel() * 4, _stream()), "tlf_paged_decode_plan")
+    return plan
+
+
 def paged_decode_attention(q, k_cache, v_cache, context_lens, block_tables, scale,
-                           k_scale=None, v_scale=None):
-    """``q [B, Hq, Dh]`` -> ``[B, Hq*Dh]``; caches ``[nblk, bs, Hkv, Dh]``."""
+                           k_scale=None, v_scale=None, plan=None):
+    """``q [B, Hq, Dh]`` -> ``[B, Hq*Dh]``; caches ``[nblk, bs, Hkv, Dh]``.  ``plan``: the output of
+    ``paged_decode_plan`` for these lengths and tables (same bits, a shorter start)."""
     lib = _lib.load()
     _need(q, BF16, "q"); _need(context_lens, torch.int32, "context_lens")
     _need(block_tables, torch.int32, "block_tables")
@@ -417,13 +434,16 @@ def paged_decode_attention(q, k_cache, v_cache, context_lens, block_tables, scal
     # sized for the largest batch so that one buffer serves every call (graph capture keeps its pointer)
     nbytes = lib.tlf_paged_decode_attn_workspace_bytes(max(B, 1024), Hq, Dh, maxb, bs)
     ws = _workspace(nbytes, q.device, "decode")
-    check(lib.tlf_paged_decode_attn(
-        q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), kv_dtype_code(k_cache),
-        k_scale.data_ptr() if k_scale is not None else None,
-        v_scale.data_ptr() if v_scale is not None else None,
-        block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(), out.data_ptr(),
-        B, Hq, Hkv, Dh, bs, maxb, nblk, float(scale), ws.data_ptr(), ws.numel(), _stream()),
-        "tlf_paged_decode_attn")
+    args = (q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), kv_dtype_code(k_cache),
+            k_scale.data_ptr() if k_scale is not None else None,
+            v_scale.data_ptr() if v_scale is not None else None,
+            block_tables.data_ptr(), block_tables.stride(0), context_lens.data_ptr(), out.data_ptr(),
+            B, Hq, Hkv, Dh, bs, maxb, nblk, float(scale), ws.data_ptr(), ws.numel())
+    if plan is None:
+        check(lib.tlf_paged_decode_attn(*args, _stream()), "tlf_paged_decode_attn")
+    else:
+        assert plan.dtype == torch.int32 and plan.device == q.device
+        check(lib.tlf_paged_decode_attn_planned(*args, plan.data_ptr(), _stream()), "tlf_paged_decode_attn_planned")
     return out
 
 

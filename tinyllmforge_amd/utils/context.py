@@ -18,6 +18,8 @@ _FIELDS = (
     ("slot_mapping", None),     # both: int32 [N] cache slot of every token of the step
     ("context_lens", None),     # decode: int32 [B] tokens per sequence, the new one included
     ("block_tables", None),     # decode, and prefill with a prefix hit: int32 [B, max blocks]
+    ("decode_plan", None),      # decode (no counterpart in the reference): the step's work split for the attention
+                                # kernel, made once by the model runner for all layers (ops.paged_decode_plan)
 )
 
 
@@ -43,14 +45,15 @@ def get_context() -> Context:
 
 
 def set_context(is_prefill, cu_seqlens_q=None, cu_seqlens_k=None, max_seqlen_q=0, max_seqlen_k=0, slot_mapping=None,
-                context_lens=None, block_tables=None):
+                context_lens=None, block_tables=None, decode_plan=None):
     """Publish one step's metadata; every argument after the first is optional, positional or by name
-    (same parameter list as tinyvllm/utils/context.py:21)."""
+    (the parameter list of tinyvllm/utils/context.py:21, then ``decode_plan``)."""
     c = _CURRENT
     c.is_prefill = is_prefill
     c.cu_seqlens_q, c.cu_seqlens_k = cu_seqlens_q, cu_seqlens_k
     c.max_seqlen_q, c.max_seqlen_k = max_seqlen_q, max_seqlen_k
     c.slot_mapping, c.context_lens, c.block_tables = slot_mapping, context_lens, block_tables
+    c.decode_plan = decode_plan
 
 
 def reset_context():
