@@ -418,3 +418,30 @@ def test_fp8_kv_cache_with_shared_prefix_end_to_end():
         llm.exit()
     agree = sum(a[0] == b[0] for a, b in zip(outs["bf16"], outs["fp8_e4m3"]))
     assert agree >= 4, f"first tokens with e4m3 KV agree with bf16 KV on only {agree} of 6 sequences"
+
+
+@pytest.mark.parametrize("eager", [False, True])
+def test_decode_plan_made_once_per_step_gives_identical_tokens(eager):
+    """Config.decode_plan: the attention kernel's work split made once per decode step (first node of the graph, or
+    one call before the layers of an eager step) against every layer scanning for itself: same tokens, with
+    sequences that end at different lengths (batch buckets change) and an e4m3 cache."""
+    from random import Random
+    from tinyllmforge_amd import LLM, SamplingParams
+    from tinyllmforge_amd.config import QWEN3_SHAPES
+    r = Random(2)
+    prompts = [[r.randint(0, 9999) for _ in range(r.randint(5, 600))] for _ in range(11)]
+    sps = [SamplingParams(temperature=0.0, ignore_eos=True, max_tokens=r.randint(2, 40)) for _ in prompts]
+    runs = []
+    for plan in (False, True):
+        llm = LLM(dict(QWEN3_SHAPES["qwen3-0.6b"], num_hidden_layers=3), max_model_len=1024, num_kvcache_blocks=40,
+                  enforce_eager=eager, seed=4, quantization="w8a16", kv_cache_dtype="fp8_e4m3", decode_plan=plan)
+        try:
+            runs.append([o["token_ids"] for o in llm.generate(prompts, sps)])
+            assert (getattr(llm.model_runner, "decode_plan_buf", None) is not None) == plan
+        finally:
+            llm.exit()
+            del llm
+            import gc
+            gc.collect()
+            torch.cuda.empty_cache()
+    assert runs[0] == runs[1] and all(len(t) == sp.max_tokens for t, sp in zip(runs[0], sps))
