@@ -391,3 +391,19 @@ def test_mfma_probe_modes_compute_the_same_sums():
     assert torch.isfinite(outs[1]).all() and not torch.equal(outs[0], outs[1])
     assert (outs[0] == outs[0].round()).all() and outs[0].min() >= 0 and outs[0].max() > 0
     assert lib.tlf_probe_mfma(out.data_ptr(), 3, 4, st) != 0          # no such mode
+
+
+def test_reduce_kernels_under_forced_split_counts():
+    """The kernels that sum the fp32 partials of a K split across workgroups load 1, 3 or 7 partials ahead and take
+    the rest in a loop; rows of 2048 ... 10240 values use 1, 2, 4 or 8 chunks per thread.  Split counts the planner
+    does not pick for these shapes are forced through TLF_GEMM_PLAN (read once per process: one child process per
+    plan, run one after the other): fused == unfused bit for bit and the plain reduce exact on integer data."""
+    import os
+    import subprocess
+    import sys
+    child = os.path.join(os.path.dirname(os.path.abspath(__file__)), "forced_split_child.py")
+    for splits in (3, 8, 16):
+        env = dict(os.environ, TLF_GEMM_PLAN="128,64,%d,4,3,1,4" % splits)
+        r = subprocess.run([sys.executable, child], env=env, capture_output=True, text=True, timeout=240)
+        assert r.returncode == 0, (splits, r.stdout[-500:], r.stderr[-500:])
+        assert "mismatches []" in r.stdout
