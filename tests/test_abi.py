@@ -51,6 +51,18 @@ def test_argument_rejection_happens_before_any_launch():
     assert lib.tlf_paged_decode_attn(16, 4096, 16, 16, 0, None, None, 16, 16, 16, 16,
                                      2, 32, 8, 64, 256, 16, 10, 0.1, None, 0, None) == -5  # Dh != 128
     assert lib.tlf_argmax_workspace_bytes(4, 151936) > 0
+    # the decode plan: NULL operands, too many sequences, a block size that is no multiple of a tile, a small buffer
+    a256 = 4096
+    nplan = lib.tlf_paged_decode_plan_bytes()
+    assert nplan > 0 and nplan % 16 == 0
+    assert lib.tlf_paged_decode_plan(None, a256, 16, 4, 256, 16, a256, nplan, None) == -1
+    assert lib.tlf_paged_decode_plan(a256, a256, 16, 1025, 256, 16, a256, nplan, None) == -2
+    assert lib.tlf_paged_decode_plan(a256, a256, 16, 4, 250, 16, a256, nplan, None) == -2
+    assert lib.tlf_paged_decode_plan(a256, a256, 8, 4, 256, 16, a256, nplan, None) == -2          # table stride < max_blocks
+    assert lib.tlf_paged_decode_plan(a256, a256, 16, 4, 256, 16, a256, nplan - 4, None) == -4
+    assert lib.tlf_paged_decode_plan(a256, a256, 16, 0, 256, 16, None, 0, None) == 0               # no sequences
+    assert lib.tlf_paged_decode_attn_planned(16, 4096, 16, 16, 0, None, None, 16, 16, 16, 16,
+                                             2, 32, 8, 128, 256, 16, 10, 0.1, a256, 1 << 30, None, None) == -1   # no plan
     # the fused entry points: NULL operands, a missing or misaligned workspace, bad shapes
     a = 4096                                                          # any 256-byte aligned non-NULL value
     assert lib.tlf_w8a16_gemm_add_rmsnorm(a, 4096, a, a, None, a, a, a, 8, 4096, 4096, 1e-6, a, 1 << 30, None) == -1
