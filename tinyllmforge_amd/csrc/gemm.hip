@@ -204,13 +204,24 @@ void gemm_dlds_kernel(const GemmParams p) {
   // eighth of x and streams W, instead of holding an eighth of W and streaming all of x (at 16384 tokens x is 6 x the
   // bytes of a 5120 x 8192 weight), and 20 tile columns, which do not divide by 8, no longer leave four XCDs with
   // half as much to do again as the other four.
-  const int xcd = blockIdx.x & 7;
-  const int local = blockIdx.x >> 3;
+  // Ownership covers the first 8 * floor(T / 8) rows (columns) of the T there are; the tiles of the remaining T % 8
+  // are dealt to the XCDs one by one after them (map_main workgroups in, consecutive workgroups sit on consecutive
+  // XCDs): an XCD with a whole extra row of tiles would finish a round of tiles after the others (50 tile rows of
+  // 256 tokens over 8 XCDs: 7 rows on two of them, 6.25 on average).
   const int walked = p.xcd_rows ? p.n_tiles : p.m_tiles;     // tiles along the dimension the XCD walks in full
-  const int per_group = p.group_n * walked;
-  const int within = local % per_group;
-  const int across = within / p.group_n;
-  const int owned = ((local / per_group) * p.group_n + within % p.group_n) * 8 + xcd;
+  int owned, across;
+  if (static_cast<int>(blockIdx.x) < p.map_main) {
+    const int xcd = blockIdx.x & 7;
+    const int local = blockIdx.x >> 3;
+    const int per_group = p.group_n * walked;
+    const int within = local % per_group;
+    across = within / p.group_n;
+    owned = ((local / per_group) * p.group_n + within % p.group_n) * 8 + xcd;
+  } else {
+    const int t = static_cast<int>(blockIdx.x) - p.map_main;
+    owned = p.map_full + t % p.map_rem;
+    across = t / p.map_rem;
+  }
   const int mt = p.xcd_rows ? owned : across;
   const int nt = p.xcd_rows ? across : owned;
   if (nt >= p.n_tiles || mt >= p.m_tiles) return;
@@ -1379,10 +1390,12 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   p.amax = nullptr;
   p.amax_parts = 0;
   p.xcd_rows = 0;
+  p.map_main = 0; p.map_full = 0; p.map_rem = 1;
   GemmPlan g;
   const bool wstream = W8 && plan_wstream(M, N, K, act, g);
   if (M <= skinny_max_m() && !wstream) {
     p.k_per_split = K; p.splits = 1; p.m_tiles = 1; p.n_tiles = 1; p.group_n = 1; p.xcd_rows = 0;
+    p.map_main = 0; p.map_full = 0; p.map_rem = 1;
     if (dry) {
       const int32_t skinny[8] = {0, 0, 0, 0, 1, 1, K, 1};  // tile 0 x 0 = the skinny kernel
       for (int i = 0; i < 8; ++i) plan_out[i] = skinny[i];
@@ -1426,24 +1439,28 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   }
   // XCD patch: group as many N-tile columns as divide this XCD's share evenly (up to 4), once
   // there are enough M-tiles for the patch to matter
-  // An XCD owns tile rows instead of tile columns (see the kernel) from 16 tile rows on, unless the columns share out
-  // over the 8 XCDs more evenly than the rows.  Measured at 8192 / 16384 tokens, us, rows / columns: 5120 x 8192
-  // 569 / 644 and 1063 / 1288, 5120 x 25600 1782 / 1967 and 3311 / 3920, 51200 x 5120 3367 / 3529 and 6744 / 7052,
-  // 10240 x 5120 676 / 706 and 1344 / 1404; the Qwen3-8B shapes 1-2 % faster; at 2048 tokens (8 tile rows) no gain.
+  // An XCD owns tile rows instead of tile columns (see the kernel) from 16 tile rows on.  Either way the rows
+  // (columns) that do not divide by 8 are dealt out tile by tile, so both forms keep the XCDs level; rows then win by
+  // the traffic: TFLOP/s rows / columns at 8192, 12800 and 16384 tokens: 10240 x 5120 1128 / 1057, 1219 / 1159,
+  // 1282 / 1251; 51200 x 5120 1293 / 1232, 1275 / 1233, 1302 / 1241; 5120 x 8192 and 5120 x 25600 within 2 %; the
+  // Qwen3-8B shapes 0 ... +4 %; at 4096 tokens (16 tile rows) -4 ... +6 %.  (With whole rows or columns per XCD 50 tile
+  // rows cost 7 rounds on two XCDs against 6.25 on average: 5120 x 8192 at 12800 tokens 1104 -> 1281 TFLOP/s.)
   // TLF_GEMM_XCD_ROWS = 0 / 1 forces the choice for tuning.
-  {
-    auto padded = [](int tiles) { return static_cast<double>((tiles + 7) / 8 * 8) / tiles; };
-    p.xcd_rows = p.m_tiles >= 16 && padded(p.m_tiles) <= padded(p.n_tiles) * 1.04;   // rows also win a tie by 4 % (less traffic)
-  }
+  p.xcd_rows = p.m_tiles >= 16;
   if (gemm_tuning().xcd_rows >= 0) p.xcd_rows = gemm_tuning().xcd_rows && p.m_tiles >= 8;
+  const int owned_total = p.xcd_rows ? p.m_tiles : p.n_tiles, walked = p.xcd_rows ? p.n_tiles : p.m_tiles;
+  const int owned_each = owned_total / 8;     // rows (columns) every XCD owns; the other owned_total % 8 are dealt out tile by tile
   {
-    const int owned = ((p.xcd_rows ? p.m_tiles : p.n_tiles) + 7) / 8;
-    if ((p.xcd_rows ? p.n_tiles : p.m_tiles) >= 8) g.group_n = owned % 4 == 0 ? 4 : owned % 3 == 0 ? 3 : owned % 2 == 0 ? 2 : 1;
-    if (gemm_tuning().group_n) g.group_n = gemm_tuning().group_n;
+    g.group_n = 1;
+    if (walked >= 8 && owned_each > 0) g.group_n = owned_each % 4 == 0 ? 4 : owned_each % 3 == 0 ? 3 : owned_each % 2 == 0 ? 2 : 1;
+    if (gemm_tuning().group_n && owned_each > 0 && owned_each % gemm_tuning().group_n == 0) g.group_n = gemm_tuning().group_n;
   }
   p.group_n = g.group_n;
-  const int owned_per_xcd = (((p.xcd_rows ? p.m_tiles : p.n_tiles) + 7) / 8 + g.group_n - 1) / g.group_n * g.group_n;
-  const dim3 grid(owned_per_xcd * 8 * (p.xcd_rows ? p.n_tiles : p.m_tiles), g.splits);
+  p.map_full = owned_each * 8;
+  p.map_rem = owned_total - p.map_full;
+  p.map_main = owned_each * 8 * walked;
+  if (p.map_rem == 0) p.map_rem = 1;          // never used then (no workgroup past map_main); keeps the kernel's % defined
+  const dim3 grid(static_cast<unsigned>(p.map_main + (owned_total - p.map_full) * walked), g.splits);
   bool launched = false;
   if constexpr (W8) {
     if (g.wstream) {

@@ -31,6 +31,9 @@ struct GemmParams {
   int32_t m_tiles, n_tiles;
   int32_t group_n;  // N-tile columns (xcd_rows: M-tile rows) walked together by one XCD
   int32_t xcd_rows; // 1: an XCD owns M-tile rows 8 c + xcd and walks all N-tile columns; 0: it owns N-tile columns
+  int32_t map_main; // workgroups of the owned part: 8 * (rows or columns per XCD) * tiles walked
+  int32_t map_full; // rows (columns) covered by ownership: a multiple of 8
+  int32_t map_rem;  // the rest of them (1 ... 7; 1 when there is none): their tiles follow, dealt out one by one
   int32_t act;      // 1: SiLU-and-mul epilogue over interleaved gate/up channels, y is [M, N/2]
                     // 2: greedy-sample epilogue, nothing but argmax keys [M, amax_parts] is stored
   unsigned long long *amax;
