@@ -407,3 +407,16 @@ def test_reduce_kernels_under_forced_split_counts():
         r = subprocess.run([sys.executable, child], env=env, capture_output=True, text=True, timeout=240)
         assert r.returncode == 0, (splits, r.stdout[-500:], r.stderr[-500:])
         assert "mismatches []" in r.stdout
+
+
+@pytest.mark.parametrize("M,N,K", [(256 * 17 + 5, 256 * 9, 256), (256 * 21 - 40, 1280, 192), (256 * 50, 256 * 3, 128),
+                                   (700, 256 * 11 + 64, 320), (3000, 2304 + 16, 64), (256 * 23, 256 * 23, 64)])
+def test_tile_rows_and_columns_that_do_not_divide_by_the_xcds_exact_on_integer_data(M, N, K):
+    """The tiled kernel deals the tile rows (from 16 rows on) or columns beyond a multiple of 8 to the XCDs tile by
+    tile: row and column counts with every kind of remainder, int8 and bf16 weights, against the exact product."""
+    from tinyllmforge_amd import ops as P
+    x = torch.randint(-3, 4, (M, K), generator=g(M)).to(BF).to(DEV)
+    w = torch.randint(-7, 8, (N, K), generator=g(N), dtype=torch.int8).to(DEV)
+    ref = ((x.double() @ w.double().T) * 0.5).to(BF)
+    assert torch.equal(P.w8a16_linear(x, w, torch.full((N,), 0.5, device=DEV)), ref)
+    assert torch.equal(P.bf16_linear(x, w.to(BF)), (x.double() @ w.double().T).to(BF))
