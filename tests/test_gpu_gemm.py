@@ -410,7 +410,8 @@ def test_reduce_kernels_under_forced_split_counts():
 
 
 @pytest.mark.parametrize("M,N,K", [(256 * 17 + 5, 256 * 9, 256), (256 * 21 - 40, 1280, 192), (256 * 50, 256 * 3, 128),
-                                   (700, 256 * 11 + 64, 320), (3000, 2304 + 16, 64), (256 * 23, 256 * 23, 64)])
+                                   (700, 256 * 11 + 64, 320), (3000, 2304 + 16, 64), (256 * 23, 256 * 23, 64),
+                                   (256 * 33 - 7, 256 * 16, 128)])
 def test_tile_rows_and_columns_that_do_not_divide_by_the_xcds_exact_on_integer_data(M, N, K):
     """The tiled kernel deals the tile rows (from 16 rows on) or columns beyond a multiple of 8 to the XCDs tile by
     tile: row and column counts with every kind of remainder, int8 and bf16 weights, against the exact product."""

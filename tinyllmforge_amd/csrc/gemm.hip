@@ -1337,6 +1337,12 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
     }
   } else if (tiles(128, 128) < 1024 && tiles(256, 128) < 256) {
     g.bn = 128; g.bm = 128; g.stages = 3; g.occ = 2; g.wn = 2;
+  } else if (!w8 && ktiles <= 64 && tiles(256, 256) >= 512 && (M + 255) / 256 * 256 * 20 <= M * 23) {
+    // bf16 weights, two rounds of 256 x 256 tiles or more, K up to 4096: the eight-wave 256 x 256 tile with two LDS
+    // stages (a bf16 K-tile of it is 64 KB; three stages do not fit).  TFLOP/s against the 256 x 128 tile at 8192 /
+    // 16384 tokens: 6144 x 4096 1125 / 1207 against 944 / 1102, 4096 x 4096 1272 / 1252 against 1117 / 1157,
+    // 24576 x 4096 1196 / 1189 against 1109 / 1122; 4096 x 12288 (192 K-tiles) ties or loses 1-3 %, hence the bound on K.
+    g.bn = 256; g.bm = 256; g.stages = 2; g.occ = 2; g.wn = 8;
   } else {  // bf16, one 256 x 128 tile per CU or more (measured 7-10 % faster than 128 x 128 from there on)
     g.bn = 256; g.bm = 128; g.stages = 3; g.occ = 1;
   }
@@ -1506,6 +1512,7 @@ int launch_gemm(const void *x, int64_t x_stride, const void *w, const float *sca
   TLF_TILE(128, 160, 4, 1, 3, 2)
   TLF_TILE(128, 192, 4, 1, 3, 2)
   TLF_TILE(128, 224, 4, 1, 3, 2)
+  TLF_TILE(256, 256, 8, 1, 2, 2)   // two stages: the bf16 form of the eight-wave 256 x 256 tile (128 KB of LDS)
   if constexpr (W8) {  // these fit LDS with int8 weights only
     TLF_TILE_KG(64, 96, 2, 1, 3, 2, 2)   // one M-tile, 64 channels, two sets of two waves
     TLF_TILE_KG(64, 128, 2, 1, 3, 2, 2)
