@@ -730,7 +730,7 @@ def cpu_baseline_e2e(llm, prompts, nseq=3, out_tokens=6):
     from oracle.model import OracleQwen3, greedy_generate
     torch.set_num_threads(os.cpu_count() if (os.cpu_count() or 0) <= 64 else 16)
     cfg = vars(llm.config.hf_config)
-    params = {k: v.data.cpu() for k, v in llm.model_runner.model.named_parameters()}
+    params = {k: v.cpu() for k, v in llm.model_runner.model.checkpoint_parameters().items()}
     model = OracleQwen3(cfg, params, exact=False)
     sample = prompts[:nseq]
     t0 = time.perf_counter()

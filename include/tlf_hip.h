@@ -251,6 +251,9 @@ int tlf_bf16_gemm(const void *x, int64_t x_stride, const void *w, void *y,
  * Needs no workspace (K is never split across workgroups).  Other constraints as tlf_w8a16_gemm. */
 int tlf_w8a16_gemm_silu_mul(const void *x, int64_t x_stride, const void *wq, const float *scale,
                             void *y, int32_t M, int32_t N, int32_t K, void *stream);
+/* The same with bf16 weights: w bf16 [N, K] row-major with its rows interleaved the same way (no scale). */
+int tlf_bf16_gemm_silu_mul(const void *x, int64_t x_stride, const void *w, void *y,
+                           int32_t M, int32_t N, int32_t K, void *stream);
 
 /* Row-parallel projection fused with what follows it in a decoder layer: replaces
  * RowParallelLinear.forward (layers/linear.py:181-183; o_proj, down_proj) followed by

@@ -251,6 +251,25 @@ def test_w8a16_gemm_fused_silu_mul_equals_the_two_kernels(M, N, K):
     assert rel <= 2e-3, rel
 
 
+@pytest.mark.parametrize("M,N,K", [(1, 6144, 1024), (16, 2048, 4096), (130, 24576, 1024), (300, 6144, 2048),
+                                   (2048, 4096, 512), (33, 272, 64), (2100, 24576, 128), (150, 24592, 256),
+                                   (8, 24576, 4096), (256 * 33, 256 * 16, 128)])
+def test_bf16_gemm_fused_silu_mul_equals_the_two_kernels(M, N, K):
+    """The bf16 gate_up projection + SiLU-and-mul in one kernel (interleaved weight rows): the bits of the plain
+    bf16 GEMM on the weight in checkpoint order followed by the activation kernel, within tolerance of the oracle."""
+    from tinyllmforge_amd import ops as P
+    x = torch.randn(M, K, generator=g(M + 9)).to(BF)
+    w = (torch.randn(N, K, generator=g(N + 1)) * 0.05).to(BF)              # checkpoint order: [gate; up]
+    wi = w[P.gate_up_interleave_index(N)].contiguous()
+    fused = P.bf16_linear_silu_mul(x.to(DEV), wi.to(DEV))
+    assert fused.shape == (M, N // 2) and fused.dtype == BF
+    two = P.silu_and_mul(P.bf16_linear(x.to(DEV), w.to(DEV)))
+    assert torch.equal(fused.view(torch.int16), two.view(torch.int16))
+    ref = O.silu_and_mul(O.linear_exact(x, w).to(BF))
+    rel = ((fused.float().cpu() - ref.float()).norm() / ref.float().norm().clamp_min(1e-6)).item()
+    assert rel <= 2e-3, rel
+
+
 @pytest.mark.parametrize("M,N,K,w8,path", [
     (120, 4096, 4096, True, "fused"), (160, 4096, 12288, True, "fused"), (97, 1024, 3072, True, "fused"),
     (120, 4096, 4096, False, "fused"), (70, 8704, 8192, True, "fused"), (50, 256, 8192, True, "fused"),

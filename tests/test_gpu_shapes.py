@@ -282,7 +282,7 @@ def run_width_check(llm, oracle, session, prompts, steps, cached=None):
 
 
 def cpu_params(llm):
-    return {k: v.data.cpu() for k, v in llm.model_runner.model.named_parameters()}
+    return {k: v.cpu() for k, v in llm.model_runner.model.checkpoint_parameters().items()}
 
 
 def random_prompts(lens, seed, vocab=151936):

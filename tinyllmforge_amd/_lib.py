@@ -44,6 +44,7 @@ SIGNATURES = {
     "tlf_w8a16_gemm": (c_int32, [_P, _I64, _P, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),
     "tlf_bf16_gemm": (c_int32, [_P, _I64, _P, _P, _I32, _I32, _I32, _P, _SZ, _P]),
     "tlf_w8a16_gemm_silu_mul": (c_int32, [_P, _I64, _P, _P, _P, _I32, _I32, _I32, _P]),
+    "tlf_bf16_gemm_silu_mul": (c_int32, [_P, _I64, _P, _P, _I32, _I32, _I32, _P]),
     "tlf_gemm_plan": (c_int32, [_I32, _I32, _I32, _I32, _P]),
     "tlf_gemm_add_rmsnorm_workspace_bytes": (_SZ, [_I32, _I32, _I32]),
     "tlf_gemm_argmax_workspace_bytes": (_SZ, [_I32, _I32, _I32]),

@@ -1711,6 +1711,15 @@ extern "C" int tlf_w8a16_gemm_silu_mul(const void *x, int64_t x_stride, const vo
                            static_cast<hipStream_t>(stream), nullptr, 1);
 }
 
+extern "C" int tlf_bf16_gemm_silu_mul(const void *x, int64_t x_stride, const void *w, void *y, int32_t M,
+                                      int32_t N, int32_t K, void *stream) {
+  if (M == 0) return TLF_OK;
+  const int rc = check_gemm_args(x, x_stride, w, y, M, N, K);
+  if (rc != TLF_OK) return rc;
+  return launch_gemm<false>(x, x_stride, w, nullptr, y, M, N, K, nullptr, 0, static_cast<hipStream_t>(stream),
+                            nullptr, 1);
+}
+
 extern "C" size_t tlf_gemm_add_rmsnorm_workspace_bytes(int32_t M, int32_t N, int32_t K) {
   if (M <= 0 || N <= 0 || K <= 0 || K % kBK) return 0;
   return align256(static_cast<size_t>(M) * N * 2) + align256(tlf_w8a16_gemm_workspace_bytes(M, N, K));

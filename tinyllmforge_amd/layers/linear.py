@@ -138,13 +138,31 @@ class MergedColumnParallelLinear(ColumnParallelLinear):
         return self
 
     def interleave_(self):
+        """Rows into the order the fused projection + SiLU-and-mul kernels read (int8 weight and scale, or the bf16
+        weight): once, after loading."""
         if not getattr(self, "interleaved", False) and len(self.output_sizes) == 2 \
                 and self.output_sizes[0] == self.output_sizes[1] \
                 and sum(self.output_sizes) % 16 == 0 and self.bias is None:
-            idx = ops.gate_up_interleave_index(sum(self.output_sizes), self.qweight.device)
-            self.qweight = self.qweight[idx].contiguous()
-            self.qscale = self.qscale[idx].contiguous()
+            if self.is_quantized:
+                if self.qweight is None:
+                    return                   # already packed without the interleave: leave it alone
+                idx = ops.gate_up_interleave_index(sum(self.output_sizes), self.qweight.device)
+                self.qweight = self.qweight[idx].contiguous()
+                self.qscale = self.qscale[idx].contiguous()
+            else:
+                idx = ops.gate_up_interleave_index(sum(self.output_sizes), self.weight.device)
+                self.weight.data = self.weight.data[idx].contiguous()
             self.interleaved = True
+
+    def natural_weight(self) -> torch.Tensor:
+        """The bf16 weight in checkpoint order ([gate; up]) whatever order it is held in."""
+        w = self.weight.data
+        if getattr(self, "interleaved", False) and w.numel():
+            idx = ops.gate_up_interleave_index(sum(self.output_sizes), w.device)
+            inv = torch.empty_like(idx)
+            inv[idx] = torch.arange(idx.numel(), device=idx.device)
+            w = w[inv]
+        return w
 
     def shard_rows(self, shard_id=None):
         return sum(self.output_sizes[:shard_id]) // self.tp_size, self.output_sizes[shard_id] // self.tp_size
@@ -159,12 +177,16 @@ class MergedColumnParallelLinear(ColumnParallelLinear):
         return super().forward(x)
 
     def forward_silu_mul(self, x: torch.Tensor) -> torch.Tensor:
-        """``SiluAndMul()(self(x))`` (activation.py:11-14 after linear.py:82-83), fused when quantised."""
+        """``SiluAndMul()(self(x))`` (activation.py:11-14 after linear.py:82-83), one kernel once the rows are interleaved."""
         if getattr(self, "interleaved", False):
-            return ops.w8a16_linear_silu_mul(x, self.pack_().qpacked, self.qscale)
+            if self.is_quantized:
+                return ops.w8a16_linear_silu_mul(x, self.pack_().qpacked, self.qscale)
+            return ops.bf16_linear_silu_mul(x, self.weight)
         return ops.silu_and_mul(super().forward(x))
 
     def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor, loaded_shard_id: int):
+        if getattr(self, "interleaved", False):
+            raise RuntimeError("this gate_up weight was re-ordered for the fused kernel: load weights before pack_linears_()")
         offset = sum(self.output_sizes[:loaded_shard_id]) // self.tp_size
         size = self.output_sizes[loaded_shard_id] // self.tp_size
         dst = param.data.narrow(self.tp_dim, offset, size)

@@ -172,9 +172,21 @@ class Qwen3ForCausalLM(nn.Module):
                 lin.quantize_()
         return self
 
+    def checkpoint_parameters(self):
+        """name -> tensor of every parameter with rows in checkpoint order: a bf16 gate_up weight that
+        ``pack_linears_`` re-ordered for the fused kernel is handed out as ``[gate; up]`` again."""
+        out = {k: v.data for k, v in self.named_parameters()}
+        for name, m in self.named_modules():
+            if getattr(m, "interleaved", False) and hasattr(m, "natural_weight") and (name + ".weight") in out:
+                out[name + ".weight"] = m.natural_weight()
+        return out
+
     def pack_linears_(self):
-        """int8 weights into the GEMM kernels' tile order (on the GPU, once, after loading / quantising)."""
+        """int8 weights into the GEMM kernels' tile order, and a bf16 gate_up weight into the row order of the fused
+        projection + SiLU-and-mul kernel (on the GPU, once, after loading / quantising)."""
         for m in self.modules():
+            if hasattr(m, "interleave_") and not getattr(m, "is_quantized", False) and m.weight.is_cuda:
+                m.interleave_()
             if hasattr(m, "pack_") and getattr(m, "is_quantized", False):
                 m.pack_()
         return self

@@ -294,6 +294,22 @@ def w8a16_linear_silu_mul(x, wq_interleaved, scale_interleaved):
     return y.view(*x.shape[:-1], N // 2)
 
 
+def bf16_linear_silu_mul(x, w_interleaved):
+    """``silu(gate) * up`` of the bf16 gate_up projection in one kernel; weight rows interleaved as
+    ``gate_up_interleave_index`` says.  Returns ``[..., N / 2]``; the bits of ``silu_and_mul(bf16_linear(x, w))``."""
+    lib = _lib.load()
+    _need(x, BF16, "x"); _need(w_interleaved, BF16, "w")
+    assert x.stride(-1) == 1 and w_interleaved.is_contiguous()
+    x2 = x.reshape(-1, x.shape[-1])
+    M, K = x2.shape
+    N = w_interleaved.shape[0]
+    assert w_interleaved.shape[1] == K and N % 16 == 0
+    y = torch.empty(M, N // 2, dtype=BF16, device=x.device)
+    check(lib.tlf_bf16_gemm_silu_mul(x2.data_ptr(), x2.stride(0), w_interleaved.data_ptr(), y.data_ptr(), M, N, K,
+                                     _stream()), "tlf_bf16_gemm_silu_mul")
+    return y.view(*x.shape[:-1], N // 2)
+
+
 def bf16_linear(x, w):
     lib = _lib.load()
     _need(x, BF16, "x"); _need(w, BF16, "w")
