@@ -1337,8 +1337,8 @@ inline GemmPlan plan_gemm(int M, int N, int K, bool w8) {
     }
   } else if (tiles(128, 128) < 1024 && tiles(256, 128) < 256) {
     g.bn = 128; g.bm = 128; g.stages = 3; g.occ = 2; g.wn = 2;
-  } else if (!w8 && ktiles <= 64 && tiles(256, 256) >= 512 && (M + 255) / 256 * 256 * 20 <= M * 23) {
-    // bf16 weights, two rounds of 256 x 256 tiles or more, K up to 4096: the eight-wave 256 x 256 tile with two LDS
+  } else if (!w8 && M >= 2048 && ktiles <= 64 && tiles(256, 256) >= 512 && (M + 255) / 256 * 256 * 20 <= M * 23) {
+    // bf16 weights at prefill sizes, two rounds of 256 x 256 tiles or more, K up to 4096: the eight-wave 256 x 256 tile with two LDS
     // stages (a bf16 K-tile of it is 64 KB; three stages do not fit).  TFLOP/s against the 256 x 128 tile at 8192 /
     // 16384 tokens: 6144 x 4096 1125 / 1207 against 944 / 1102, 4096 x 4096 1272 / 1252 against 1117 / 1157,
     // 24576 x 4096 1196 / 1189 against 1109 / 1122; 4096 x 12288 (192 K-tiles) ties or loses 1-3 %, hence the bound on K.
