@@ -266,3 +266,14 @@ def test_one_plan_serves_every_layer_of_a_step():
     few = P.paged_decode_plan(cl[:7].contiguous(), bt[:7].contiguous(), 256)
     bad = P.paged_decode_attention(q, kc, vc, cl, bt, 0.0884, plan=few)
     assert torch.isnan(bad.float()).all()
+
+
+def test_decode_largest_batch_the_plan_holds():
+    """1024 sequences (the most one call and one plan take) of 0 ... 89 tokens: every workgroup's share spans several
+    sequences; both entry points (run_both compares their bits) against the oracle."""
+    ge = torch.Generator().manual_seed(1)
+    ctxs = torch.randint(0, 90, (1024,), generator=ge).tolist()
+    ctxs[0], ctxs[-1] = 0, 1
+    got, ref = run_both(make_case(3, 1024, 32, 8, 16, ctxs, sum((c + 15) // 16 for c in ctxs) + 3))
+    check(got, ref)
+    assert (got[0] == 0).all()
